@@ -1,0 +1,71 @@
+"""Run-time settings of the engine (not of the model).
+
+Names and defaults follow the reference's server flags
+(v3/crates/rvllm-serve/src/lib.rs:61-79: max_model_len 8192,
+max_num_batched_tokens 2048, max_prefill_chunk 128) and its runtime limits
+(v3/crates/rvllm-core/src/config/builder.rs:61-133: block size in {16, 32, 64},
+at most 256 sequences); like the reference's builder, validation reports every
+bad field at once.  The reference serves one sequence at a time
+(lib.rs:134-136); here ``max_num_seqs`` is a real limit.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional
+
+import torch
+
+from .errors import ConfigError
+
+DTYPES = {
+    "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+    "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
+}
+PAGE_SIZES = (16, 32, 64)
+
+
+@dataclasses.dataclass
+class EngineConfig:
+    dtype: str = "bfloat16"
+    device: str = "cuda:0"
+    page_size: int = 16
+    max_model_len: int = 8192
+    max_num_seqs: int = 8
+    max_num_batched_tokens: int = 2048
+    max_prefill_chunk: int = 128
+    # Tokens the cache pool is made for; None = max_num_seqs * max_model_len.
+    max_cache_tokens: Optional[int] = None
+    # Replay decode-only steps from captured HIP graphs (bf16 only).
+    use_graphs: bool = False
+
+    @property
+    def torch_dtype(self) -> torch.dtype:
+        return DTYPES[self.dtype]
+
+    def validate(self) -> "EngineConfig":
+        problems = []
+        if self.dtype not in DTYPES:
+            problems.append(f"dtype {self.dtype!r} must be one of {sorted(set(DTYPES))}")
+        if self.page_size not in PAGE_SIZES:
+            problems.append(f"page_size {self.page_size} must be one of {PAGE_SIZES}")
+        if not 1 <= self.max_num_seqs <= 256:
+            problems.append(f"max_num_seqs {self.max_num_seqs} must be in 1..=256")
+        if self.max_model_len < 1:
+            problems.append("max_model_len must be >= 1")
+        if self.max_num_batched_tokens < 1:
+            problems.append("max_num_batched_tokens must be >= 1")
+        if self.max_prefill_chunk < 1:
+            problems.append("max_prefill_chunk must be >= 1")
+        if self.max_prefill_chunk > self.max_num_batched_tokens:
+            problems.append("max_prefill_chunk must not exceed max_num_batched_tokens")
+        if self.max_cache_tokens is not None and self.max_cache_tokens < self.page_size:
+            problems.append("max_cache_tokens must hold at least one page")
+        if problems:
+            raise ConfigError("engine configuration", problems)
+        return self
+
+    def cache_tokens(self) -> int:
+        if self.max_cache_tokens is not None:
+            return self.max_cache_tokens
+        return self.max_num_seqs * self.max_model_len

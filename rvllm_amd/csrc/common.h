@@ -1,0 +1,107 @@
+// Shared device helpers for the gfx950 kernels: storage types, wave64
+// reductions, and the error channel of the C entry points.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define RV_WAVE 64
+
+// ---------------------------------------------------------------------------
+// Error channel.  Every entry point returns 0 or a negative code and leaves a
+// message that rv_last_error() returns; it validates shapes on the host before
+// it launches anything.
+// ---------------------------------------------------------------------------
+extern "C" const char* rv_last_error();
+int rv_fail(const char* fmt, ...);
+
+#define RV_CHECK(cond, ...)                 \
+  do {                                      \
+    if (!(cond)) return rv_fail(__VA_ARGS__); \
+  } while (0)
+
+#define RV_LAUNCH_CHECK(name)                                              \
+  do {                                                                     \
+    hipError_t e_ = hipGetLastError();                                     \
+    if (e_ != hipSuccess) return rv_fail("%s: launch failed: %s", name,    \
+                                         hipGetErrorString(e_));           \
+  } while (0)
+
+// dtype codes shared with Python
+enum RvDType { RV_F32 = 0, RV_BF16 = 1 };
+
+// ---------------------------------------------------------------------------
+// bfloat16 storage: 16 bits, round to nearest even on store.
+// ---------------------------------------------------------------------------
+struct bf16_t {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float rv_to_float(float x) { return x; }
+__device__ __forceinline__ float rv_to_float(bf16_t x) {
+  return __uint_as_float(((uint32_t)x.bits) << 16);
+}
+
+__device__ __forceinline__ uint16_t rv_f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T rv_from_float(float x);
+template <>
+__device__ __forceinline__ float rv_from_float<float>(float x) {
+  return x;
+}
+template <>
+__device__ __forceinline__ bf16_t rv_from_float<bf16_t>(float x) {
+  bf16_t r;
+  r.bits = rv_f32_to_bf16_bits(x);
+  return r;
+}
+
+// Value as it reads back after a store in T.
+template <typename T>
+__device__ __forceinline__ float rv_round_to(float x) {
+  return rv_to_float(rv_from_float<T>(x));
+}
+
+// A weight vector that may be stored in either type (norm weights keep the
+// type they were stored in).
+__device__ __forceinline__ float rv_load_w(const void* w, int is_f32, int i) {
+  return is_f32 ? ((const float*)w)[i] : rv_to_float(((const bf16_t*)w)[i]);
+}
+
+// ---------------------------------------------------------------------------
+// wave64 and block reductions
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float rv_wave_sum(float v) {
+#pragma unroll
+  for (int off = RV_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, RV_WAVE);
+  return v;
+}
+__device__ __forceinline__ float rv_wave_max(float v) {
+#pragma unroll
+  for (int off = RV_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, RV_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads (16 waves).  Every thread gets the
+// result.  `scratch` holds 16 floats of LDS.  The order of the additions is
+// fixed by the block size alone.
+__device__ __forceinline__ float rv_block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (RV_WAVE - 1);
+  const int wave = threadIdx.x / RV_WAVE;
+  const int nwaves = (blockDim.x + RV_WAVE - 1) / RV_WAVE;
+  v = rv_wave_sum(v);
+  __syncthreads();  // scratch may still be read from an earlier call
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  return total;
+}
+
+static inline int rv_div_up(long long a, long long b) { return (int)((a + b - 1) / b); }

@@ -1,0 +1,139 @@
+"""The model runner: one model, its cache, and the step function.
+
+``step`` takes a batch of (request, its next tokens) — portions of prompts
+beside single decoded tokens, cut anywhere — runs exactly those tokens as one
+batch against the cache, and returns 32-bit logits at the wanted places.  It
+is the only way tokens reach the model: generation, the command line and
+trace replay all go through it.
+"""
+
+from __future__ import annotations
+
+import os
+from typing import Hashable, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, group_name
+from ..cache.storage import CacheStorage
+from ..config.engine_config import EngineConfig
+from ..kernels import ops
+from ..models.model import DecoderModel
+from ..models.registry import Architecture, get_architecture, load_config
+from ..parts.base import KVNeed
+from ..weights.loader import detect_prefix, load_tensors, open_model_files, tensor_names
+from ..weights.random_init import random_tensors
+from .batch import BatchBuilder, Portion, StepBatch
+
+# Tensors of a multimodal checkpoint that the text decoder leaves alone.
+IGNORED_TENSOR_PREFIXES = ("vision_tower.", "model.vision_tower.", "multi_modal_projector.",
+                           "model.multi_modal_projector.")
+
+
+class ModelRunner:
+    def __init__(self, model: DecoderModel, engine_config: EngineConfig):
+        """``model`` has its weights bound already."""
+        self.model = model
+        self.config = engine_config.validate()
+        self.device = model.device
+        self.dtype = model.dtype
+        cfg = self.config
+        ps = cfg.page_size
+        needs = model.cache_needs()
+        full_pages = max(1, -(-cfg.cache_tokens() // ps))
+        num_pages = {}
+        for need in needs:
+            if isinstance(need, KVNeed):
+                name = group_name(need.window)
+                if need.window is None:
+                    num_pages[name] = full_pages
+                else:
+                    # A request holds at most the window behind its portion, the
+                    # portion, and the partly filled pages at both ends.
+                    per_request = -(-(need.window - 1 + cfg.max_num_batched_tokens) // ps) + 1
+                    num_pages[name] = min(full_pages, cfg.max_num_seqs * per_request)
+        self.cache = CacheManager(needs, ps, num_pages, cfg.max_num_seqs)
+        self.storage = CacheStorage(self.cache, self.device, self.dtype)
+        width = -(-cfg.max_model_len // ps)
+        self.builder = BatchBuilder(self.device, cfg.max_num_batched_tokens, cfg.max_num_seqs,
+                                    {name: width for name in self.cache.groups})
+
+    # ---- construction --------------------------------------------------
+    @classmethod
+    def from_model_dir(cls, model_dir: str | os.PathLike, engine_config: EngineConfig) -> "ModelRunner":
+        """Model class by config.json, weights by name from the folder's safetensors."""
+        engine_config.validate()
+        ops.library()  # fail now, and loudly, if the kernels cannot be built or loaded
+        arch, config = load_config(model_dir)
+        files = open_model_files(model_dir)
+        try:
+            prefix = detect_prefix(tensor_names(files))
+            model = DecoderModel(arch.build_spec(config, prefix))
+            tensors = load_tensors(files, model.param_specs(), engine_config.torch_dtype, source=str(model_dir),
+                                   ignore=IGNORED_TENSOR_PREFIXES)
+            model.bind(tensors, engine_config.device, engine_config.torch_dtype)
+        finally:
+            for f in files:
+                f.close()
+        return cls(model, engine_config)
+
+    @classmethod
+    def from_random(cls, config, seed: int, engine_config: EngineConfig) -> "ModelRunner":
+        """Random weights made on the device (no folder is written)."""
+        engine_config.validate()
+        ops.library()
+        arch = get_architecture(config.architecture)
+        model = DecoderModel(arch.build_spec(config))
+        tensors = random_tensors(model.param_specs(), seed, engine_config.device, engine_config.torch_dtype)
+        model.bind(tensors, engine_config.device, engine_config.torch_dtype)
+        return cls(model, engine_config)
+
+    # ---- requests ----------------------------------------------------
+    def add_request(self, request: Hashable) -> None:
+        rc = self.cache.add_request(request)
+        self.storage.clear_slot(rc.slot)
+
+    def release(self, request: Hashable) -> None:
+        self.cache.release(request)
+
+    def length(self, request: Hashable) -> int:
+        return self.cache.length(request)
+
+    # ---- the step ------------------------------------------------------
+    def step(self, entries: Sequence[tuple[Hashable, Sequence[int], Sequence[int]]]) -> torch.Tensor:
+        """``entries``: (request, next tokens, wanted places among them).
+
+        Runs only these tokens, as one batch, from the cache that earlier
+        steps left; returns float32 logits ``[number of wanted places, vocab]``
+        in the order of the entries and of their wanted places.  Raises
+        ``OutOfPages`` before anything ran if the cache cannot hold the
+        tokens."""
+        if not entries:
+            return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32, device=self.device)
+        vocab = self.model.spec.vocab_size
+        portions = []
+        seen = set()
+        for request, tokens, want in entries:
+            if request in seen:
+                raise ValueError(f"request {request!r} appears twice in one step")
+            seen.add(request)
+            start = self.cache.length(request)
+            if start + len(tokens) > self.config.max_model_len:
+                raise ValueError(f"request {request!r} would hold {start + len(tokens)} tokens, "
+                                 f"max_model_len is {self.config.max_model_len}")
+            ids = np.asarray(tokens, dtype=np.int64)
+            if ids.ndim != 1 or ids.size == 0:
+                raise ValueError(f"request {request!r}: a portion must hold at least one token")
+            if ids.min() < 0 or ids.max() >= vocab:
+                raise ValueError(f"request {request!r}: token id outside the vocabulary of {vocab}")
+            portions.append(Portion(request, ids, start, want))
+        self.cache.require([(p.request, p.start + len(p.tokens)) for p in portions])
+        for p in portions:
+            self.cache.extend(p.request, p.start + len(p.tokens))
+        tables = {name: [self.cache.table(p.request, name) for p in portions] for name in self.cache.groups}
+        batch = self.builder.build(portions, tables, [self.cache.slot(p.request) for p in portions])
+        logits = self.model.forward(batch, self.storage.views)
+        for p in portions:
+            self.cache.commit(p.request, p.start + len(p.tokens))
+        return logits

@@ -1,0 +1,286 @@
+"""Python face of the HIP kernels.
+
+Every function takes torch tensors that live on the GPU, checks their shapes
+and types on the host, and launches on torch's current stream, so the calls
+can be captured in a HIP graph.  Nothing here computes on the CPU or falls
+back to a library: if the kernel library cannot be loaded the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+_lib = None
+_lock = threading.Lock()
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def library():
+    """The loaded kernel library; builds it when no current build exists."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                path = _build.ensure_built()
+                try:
+                    lib = ctypes.CDLL(str(path))
+                except OSError as e:  # pragma: no cover
+                    raise KernelError(f"cannot load the kernel library {path}: {e}") from e
+                lib.rv_last_error.restype = ctypes.c_char_p
+                _lib = lib
+    return _lib
+
+
+def library_path() -> Optional[str]:
+    p = _build.find_library()
+    return str(p) if p else None
+
+
+def _check(code: int) -> None:
+    if code != 0:
+        raise KernelError(library().rv_last_error().decode())
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {t.dtype}; kernels take float32 and bfloat16") from None
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel arguments must live on the GPU")
+            _need(t.is_contiguous(), "kernel arguments must be contiguous")
+
+
+def _i32(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        _need(t.dtype == torch.int32, f"index tensors must be int32, got {t.dtype}")
+
+
+_c_int, _c_float, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_longlong
+
+
+# --------------------------------------------------------------------------
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, scale: float, out: torch.Tensor) -> torch.Tensor:
+    _gpu(table, ids, out)
+    _i32(ids)
+    vocab, hidden = table.shape
+    n = ids.numel()
+    _need(out.shape == (n, hidden), f"embed_gather: out is {tuple(out.shape)}, expected {(n, hidden)}")
+    _check(library().rv_embed_gather(_stream(), _ptr(table), _dt(table), _ptr(ids), _ptr(out), _dt(out), _c_int(n),
+                                     _c_int(hidden), _c_int(vocab), _c_float(scale)))
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float,
+            out: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Row-wise RMSNorm.  With ``rows`` (int32 indices into the rows of a 2-d
+    ``x``, all in range: the caller built them) output row r is the norm of
+    x[rows[r]]."""
+    width = x.shape[-1]
+    if rows is not None:
+        _need(x.dim() == 2, "rmsnorm: a row index needs a 2-d input")
+        _i32(rows)
+        n_rows = rows.numel()
+        if out is None:
+            out = torch.empty((n_rows, width), dtype=x.dtype, device=x.device)
+        _need(out.shape == (n_rows, width) and out.dtype == x.dtype, "rmsnorm: bad out")
+    else:
+        n_rows = x.numel() // width
+        if out is None:
+            out = torch.empty_like(x)
+        _need(out.shape == x.shape and out.dtype == x.dtype, "rmsnorm: out must match x")
+    _gpu(x, weight, out, rows)
+    _need(weight.shape == (width,), f"rmsnorm: weight is {tuple(weight.shape)}, expected ({width},)")
+    _check(library().rv_rmsnorm(_stream(), _ptr(x), _ptr(rows), _ptr(weight), _c_int(weight.dtype == torch.float32),
+                                _ptr(out), _dt(x), _c_int(n_rows), _c_int(width), _c_float(eps), _c_float(offset)))
+    return out
+
+
+def add_rmsnorm(branch: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, residual: torch.Tensor,
+                next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0, next_offset: float = 0.0,
+                next_out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """residual += rmsnorm(branch); with ``next_weight`` also returns rmsnorm(residual)."""
+    _gpu(branch, weight, residual, next_weight, next_out)
+    width = branch.shape[-1]
+    rows = branch.numel() // width
+    _need(residual.shape == branch.shape and residual.dtype == branch.dtype, "add_rmsnorm: residual must match branch")
+    _need(weight.shape == (width,), "add_rmsnorm: bad weight shape")
+    if next_weight is not None:
+        _need(next_weight.shape == (width,), "add_rmsnorm: bad next weight shape")
+        if next_out is None:
+            next_out = torch.empty_like(residual)
+        _need(next_out.shape == residual.shape and next_out.dtype == residual.dtype, "add_rmsnorm: bad next_out")
+    _check(library().rv_add_rmsnorm(
+        _stream(), _ptr(branch), _ptr(weight), _c_int(weight.dtype == torch.float32), _ptr(residual),
+        _ptr(next_weight), _c_int(next_weight is not None and next_weight.dtype == torch.float32),
+        _ptr(next_out if next_weight is not None else None), _dt(branch), _c_int(rows), _c_int(width), _c_float(eps),
+        _c_float(offset), _c_float(next_eps), _c_float(next_offset)))
+    return next_out if next_weight is not None else None
+
+
+ACTIVATIONS = {"gelu_pytorch_tanh": 0, "gelu_tanh": 0, "silu": 1}
+
+
+def gated_act(gate_up: torch.Tensor, activation: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]"""
+    _gpu(gate_up, out)
+    rows, two_i = gate_up.shape
+    _need(two_i % 2 == 0, "gated_act: width must be even")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((rows, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _need(out.shape == (rows, inter) and out.dtype == gate_up.dtype, "gated_act: bad out")
+    _need(activation in ACTIVATIONS, f"gated_act: unknown activation {activation!r}")
+    _check(library().rv_gated_act(_stream(), _ptr(gate_up), _ptr(out), _dt(gate_up), _c_int(rows), _c_int(inter),
+                                  _c_int(ACTIVATIONS[activation])))
+    return out
+
+
+def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    _gpu(logits)
+    _need(logits.dtype == torch.float32, "softcap: logits must be float32")
+    _check(library().rv_softcap(_stream(), _ptr(logits), _c_ll(logits.numel()), _c_float(cap)))
+    return logits
+
+
+def gemm_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T with 32-bit multiply-adds."""
+    _need(a.is_cuda and w.is_cuda and out.is_cuda, "gemm: arguments must live on the GPU")
+    _need(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm: matrices expected")
+    m, k = a.shape
+    n, k2 = w.shape
+    _need(k == k2, f"gemm: inner sizes differ: {k} vs {k2}")
+    _need(out.shape == (m, n), f"gemm: out is {tuple(out.shape)}, expected {(m, n)}")
+    _need(a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "gemm: rows must be contiguous")
+    _check(library().rv_gemm_plain(_stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), _c_int(m),
+                                   _c_int(n), _c_int(k), _c_ll(a.stride(0) if m > 1 else k),
+                                   _c_ll(w.stride(0) if n > 1 else k), _c_ll(out.stride(0) if m > 1 else n)))
+    return out
+
+
+def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Optional[torch.Tensor],
+                          k_weight: Optional[torch.Tensor], eps: float, offset: float,
+                          inv_freq: Optional[torch.Tensor], rotary_dim: int, positions: torch.Tensor,
+                          token_req: torch.Tensor, block_table: Optional[torch.Tensor],
+                          k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], num_q_heads: int,
+                          num_kv_heads: int, head_dim: int, write_kv: bool = True) -> torch.Tensor:
+    _gpu(qkv, q_out, q_weight, k_weight, inv_freq, positions, token_req, block_table, k_pages, v_pages)
+    _i32(positions, token_req)
+    n = qkv.shape[0]
+    _need(qkv.shape == (n, (num_q_heads + 2 * num_kv_heads) * head_dim), "qk_norm_rope: bad qkv shape")
+    _need(q_out.shape == (n, num_q_heads * head_dim) and q_out.dtype == qkv.dtype, "qk_norm_rope: bad q_out")
+    _need(positions.numel() >= n and token_req.numel() >= n, "qk_norm_rope: positions/token_req too short")
+    w_f32 = 0
+    if q_weight is not None:
+        _need(k_weight is not None and q_weight.shape == (head_dim,) and k_weight.shape == (head_dim,),
+              "qk_norm_rope: bad norm weights")
+        _need(q_weight.dtype == k_weight.dtype, "qk_norm_rope: norm weights must share a dtype")
+        w_f32 = int(q_weight.dtype == torch.float32)
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() >= rotary_dim // 2, "qk_norm_rope: bad inv_freq")
+    page_size = num_pages = width = 0
+    if write_kv:
+        _need(k_pages is not None and v_pages is not None and block_table is not None, "qk_norm_rope: no cache given")
+        _i32(block_table)
+        num_pages, page_size, nkv, hd = k_pages.shape
+        _need((nkv, hd) == (num_kv_heads, head_dim) and v_pages.shape == k_pages.shape, "qk_norm_rope: bad page shape")
+        _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "qk_norm_rope: cache dtype differs")
+        width = block_table.shape[1]
+    _check(library().rv_qk_norm_rope_kv_write(
+        _stream(), _ptr(qkv), _ptr(q_out), _ptr(q_weight), _ptr(k_weight), _c_int(w_f32), _c_float(eps),
+        _c_float(offset), _ptr(inv_freq), _c_int(rotary_dim if inv_freq is not None else 0), _ptr(positions),
+        _ptr(token_req), _ptr(block_table), _c_int(width), _ptr(k_pages), _ptr(v_pages), _c_int(page_size),
+        _c_int(num_pages), _dt(qkv), _c_int(n), _c_int(num_q_heads), _c_int(num_kv_heads), _c_int(head_dim),
+        _c_int(int(write_kv))))
+    return q_out
+
+
+def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                            positions: torch.Tensor, token_req: torch.Tensor, out: torch.Tensor, num_q_heads: int,
+                            scale: float, window: Optional[int]) -> torch.Tensor:
+    _gpu(q, k_pages, v_pages, block_table, positions, token_req, out)
+    _i32(block_table, positions, token_req)
+    n = q.shape[0]
+    num_pages, page_size, nkv, hd = k_pages.shape
+    _need(q.shape == (n, num_q_heads * hd), f"attention: q is {tuple(q.shape)}, expected {(n, num_q_heads * hd)}")
+    _need(out.shape == q.shape and out.dtype == q.dtype, "attention: out must match q")
+    _need(v_pages.shape == k_pages.shape and k_pages.dtype == q.dtype and v_pages.dtype == q.dtype,
+          "attention: cache must match q")
+    _need(positions.numel() >= n and token_req.numel() >= n, "attention: positions/token_req too short")
+    _check(library().rv_paged_attention_generic(
+        _stream(), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _c_int(block_table.shape[1]),
+        _ptr(positions), _ptr(token_req), _ptr(out), _dt(q), _c_int(n), _c_int(num_q_heads), _c_int(nkv), _c_int(hd),
+        _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_float(scale)))
+    return out
+
+
+def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, step,
+                    out: torch.Tensor, num_q_heads: int, scale: float, window: Optional[int]) -> torch.Tensor:
+    """Attention of the step's tokens over the cache; picks the kernel.
+
+    The 32-bit path always runs the generic kernel.  bf16 runs the
+    matrix-core kernels where one covers the head size, else the generic one."""
+    return paged_attention_generic(q, k_pages, v_pages, block_table, step.positions, step.token_req, out,
+                                   num_q_heads, scale, window)
+
+
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _gpu(logits, out)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "argmax: float32 [rows, vocab] expected")
+    rows, vocab = logits.shape
+    if out is None:
+        out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    parts = library().rv_argmax_parts(_c_int(vocab))
+    ws_val = torch.empty(rows * parts, dtype=torch.float32, device=logits.device)
+    ws_idx = torch.empty(rows * parts, dtype=torch.int32, device=logits.device)
+    _check(library().rv_argmax(_stream(), _ptr(logits), _c_int(rows), _c_int(vocab), _c_ll(vocab), _ptr(ws_val),
+                               _ptr(ws_idx), _ptr(out)))
+    return out
+
+
+def topk_select(logits: torch.Tensor, k: int, inv_temp: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """The k largest logits of every row, times 1/T, with their ids (unordered)."""
+    _gpu(logits, inv_temp)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "topk_select: float32 [rows, vocab] expected")
+    rows, vocab = logits.shape
+    _need(inv_temp.dtype == torch.float32 and inv_temp.numel() == rows, "topk_select: one 1/T per row expected")
+    vals = torch.empty((rows, k), dtype=torch.float32, device=logits.device)
+    idx = torch.empty((rows, k), dtype=torch.int32, device=logits.device)
+    _check(library().rv_topk_select(_stream(), _ptr(logits), _c_int(rows), _c_int(vocab), _c_ll(vocab), _c_int(k),
+                                    _ptr(inv_temp), _ptr(vals), _ptr(idx)))
+    return vals, idx
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optional[torch.Tensor]:
+    """out = x @ w^T on the matrix cores for bf16 inputs; None when no
+    hand-written kernel covers the shape (the caller then uses another path)."""
+    return None

@@ -1,0 +1,180 @@
+"""Interfaces of the parts a layer is put together from.
+
+A part gets its sizes and constants through its ``PartSpec``; it never sees a
+model configuration or knows which model it is in.  A part says which tensors
+it wants (``param_specs``), takes them (``bind``) and runs on the tokens of
+one step (``forward``).  What a mixer keeps between steps it declares as a
+``CacheNeed``; the cache manager groups layers by need.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import TYPE_CHECKING, Optional, Sequence
+
+import torch
+
+if TYPE_CHECKING:  # pragma: no cover
+    from ..engine.batch import StepBatch
+
+
+# --------------------------------------------------------------------------
+# Parameters
+# --------------------------------------------------------------------------
+@dataclasses.dataclass(frozen=True)
+class ParamSpec:
+    """One tensor a part reads from the checkpoint.
+
+    ``init`` tells the random-weights mode how to fill it: ``("normal", std)``
+    for floating tensors, ``("randint", lo, hi)`` for integer tables."""
+
+    name: str
+    shape: tuple[int, ...]
+    init: tuple = ("normal", 0.02)
+    integer: bool = False
+
+
+class Part:
+    """Base of every part."""
+
+    def param_specs(self, prefix: str) -> list[ParamSpec]:
+        return []
+
+    def bind(self, tensors: dict[str, torch.Tensor], prefix: str, device: torch.device, dtype: torch.dtype) -> None:
+        """Take the tensors named by ``param_specs(prefix)``.  ``dtype`` is the
+        dtype of activations; a part may fuse or re-lay tensors here."""
+
+
+# --------------------------------------------------------------------------
+# What a mixer keeps between steps
+# --------------------------------------------------------------------------
+@dataclasses.dataclass(frozen=True)
+class KVNeed:
+    """Keys and values of earlier tokens, in pages.
+
+    ``window`` is None when every earlier token stays visible, else the
+    number of most recent positions (the current one included) a token can
+    see.  Layers with the same ``window`` share a page group and block table;
+    head counts and sizes may differ between them."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclasses.dataclass(frozen=True)
+class StateNeed:
+    """A state of fixed size for every live request (one slot each)."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+CacheNeed = "KVNeed | StateNeed | None"
+
+
+@dataclasses.dataclass
+class KVCacheView:
+    """What an attention-like mixer gets for its layer: the key and value
+    pages ``[num_pages, page_size, num_kv_heads, head_dim]`` and the name of
+    the group whose block table addresses them.  ``writes`` is False for a
+    layer that reads another layer's cache."""
+
+    k_pages: torch.Tensor
+    v_pages: torch.Tensor
+    group: str
+    page_size: int
+    writes: bool = True
+
+    def reader(self) -> "KVCacheView":
+        return dataclasses.replace(self, writes=False)
+
+
+@dataclasses.dataclass
+class StateView:
+    """What a mixer with fixed-size state gets: ``[num_slots, *shape]``; the
+    step batch tells the slot of each request.  A request's slot is zeroed
+    when it is handed out."""
+
+    slots: torch.Tensor
+    writes: bool = True
+
+    def reader(self) -> "StateView":
+        return dataclasses.replace(self, writes=False)
+
+
+# --------------------------------------------------------------------------
+# Parts
+# --------------------------------------------------------------------------
+class Norm(Part):
+    """y = norm(x) over the last dimension."""
+
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+    def forward_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        """norm(x[rows]) for an int32 index tensor."""
+        return self.forward(x.index_select(0, rows.long()))
+
+    def add_into(
+        self,
+        branch: torch.Tensor,
+        residual: torch.Tensor,
+        then: "Optional[Norm]" = None,
+        then_out: Optional[torch.Tensor] = None,
+    ) -> Optional[torch.Tensor]:
+        """residual += norm(branch), in place; when ``then`` is given also
+        return then(residual).  The default runs the pieces one by one; a norm
+        with a fused kernel overrides it."""
+        normed = self.forward(branch)
+        residual.add_(normed)
+        return then.forward(residual, out=then_out) if then is not None else None
+
+
+class PositionEncoding(Part):
+    """How a mixer marks positions.  ``kernel_args`` gives what the fused
+    query/key kernel needs: the number of rotated dimensions and the table of
+    inverse frequencies (already divided by any scaling factor)."""
+
+    rotary_dim: int = 0
+
+    def inv_freq(self, device: torch.device) -> Optional[torch.Tensor]:
+        return None
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request."""
+
+    def cache_need(self):
+        return None
+
+    def forward(self, x: torch.Tensor, step: "StepBatch", cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """Works on every token alone."""
+
+    def forward(self, x: torch.Tensor, step: "StepBatch") -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """The arrangement of norm, mixer, feed-forward and the residual sum in
+    one layer.  ``forward`` updates the residual stream ``x`` in place.
+
+    ``entry_norm`` is the norm the block applies to the residual stream first,
+    or None.  ``forward`` may be given that norm's output (``entered``) when
+    the block before has computed it, and may be asked to return
+    ``then(x)`` for the block after; a block that does not fuse returns None
+    and the caller applies the norm itself."""
+
+    mixer: Mixer
+    feed_forward: FeedForward
+
+    def entry_norm(self) -> Optional[Norm]:
+        return None
+
+    def forward(self, x: torch.Tensor, step: "StepBatch", cache, entered: Optional[torch.Tensor] = None,
+                then: Optional[Norm] = None) -> Optional[torch.Tensor]:
+        raise NotImplementedError

@@ -1,0 +1,101 @@
+"""The tiny configurations the tests run on.  A and B differ in every size and
+option: layers 2 / 3, kinds given by layer_types / by sliding_window_pattern,
+window 8 / 5, hidden 64 / 96, heads 4:2 / 6:3, head size 16 / 32 (query width
+equal to / different from hidden), intermediate 128 / 160, vocabulary 256 (a
+power of two) / 509 (a prime), global base 1e6 / 5e5, no scaling / linear 4,
+score scalar equal to / different from the head size, eps 1e-6 / 1e-5.
+C has the head size of the large models (256), one key/value head and a
+soft-cap.
+"""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+
+import torch
+
+CONFIG_A = {
+    "architectures": ["Gemma3ForCausalLM"],
+    "num_hidden_layers": 2,
+    "layer_types": ["sliding_attention", "full_attention"],
+    "hidden_size": 64,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 2,
+    "head_dim": 16,
+    "intermediate_size": 128,
+    "vocab_size": 256,
+    "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 4096,
+    "sliding_window": 8,
+    "rope_theta": 1000000.0,
+    "rope_local_base_freq": 10000.0,
+    "rope_scaling": None,
+    "query_pre_attn_scalar": 16,
+    "hidden_activation": "gelu_pytorch_tanh",
+    "tie_word_embeddings": True,
+    "final_logit_softcapping": None,
+    "attn_logit_softcapping": None,
+}
+
+CONFIG_B = {
+    "architectures": ["Gemma3ForCausalLM"],
+    "num_hidden_layers": 3,
+    "sliding_window_pattern": 3,
+    "hidden_size": 96,
+    "num_attention_heads": 6,
+    "num_key_value_heads": 3,
+    "head_dim": 32,
+    "intermediate_size": 160,
+    "vocab_size": 509,
+    "rms_norm_eps": 1e-5,
+    "max_position_embeddings": 2048,
+    "sliding_window": 5,
+    "rope_theta": 500000.0,
+    "rope_local_base_freq": 10000.0,
+    "rope_scaling": {"rope_type": "linear", "factor": 4.0},
+    "query_pre_attn_scalar": 48,
+    "hidden_activation": "gelu_pytorch_tanh",
+    "tie_word_embeddings": True,
+    "final_logit_softcapping": None,
+}
+
+CONFIG_C = {
+    "architectures": ["Gemma3ForCausalLM"],
+    "num_hidden_layers": 2,
+    "layer_types": ["full_attention", "sliding_attention"],
+    "hidden_size": 80,
+    "num_attention_heads": 2,
+    "num_key_value_heads": 1,
+    "head_dim": 256,
+    "intermediate_size": 112,
+    "vocab_size": 300,
+    "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 4096,
+    "sliding_window": 70,
+    "rope_theta": 1000000.0,
+    "rope_local_base_freq": 10000.0,
+    "rope_scaling": {"rope_type": "linear", "factor": 8.0},
+    "query_pre_attn_scalar": 256,
+    "hidden_activation": "gelu_pytorch_tanh",
+    "tie_word_embeddings": True,
+    "final_logit_softcapping": 30.0,
+}
+
+CONFIGS = {"A": (CONFIG_A, 0), "B": (CONFIG_B, 1), "C": (CONFIG_C, 2)}
+
+
+def write_model(folder, name: str, dtype=torch.bfloat16, seed=None) -> Path:
+    """Write config ``name`` with random weights into ``folder`` through the
+    framework's random-weights mode; returns the folder."""
+    from rvllm_amd.models.registry import architecture_of
+    import rvllm_amd.models.gemma3  # noqa: F401  (registers the architecture)
+    from rvllm_amd.weights.random_init import write_random_model
+
+    doc, default_seed = CONFIGS[name]
+    arch = architecture_of(doc)
+    config = arch.read_config(doc, f"tiny config {name}")
+    out = write_random_model(Path(folder), config, default_seed if seed is None else seed, dtype)
+    # keep the document as written above, so that each spelling of the keys is read
+    (out / "config.json").write_text(json.dumps(doc, indent=2))
+    return out
