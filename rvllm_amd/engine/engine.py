@@ -1,0 +1,119 @@
+"""The engine: scheduler, model runner and sampler in one loop.
+
+    engine = LLMEngine.from_model_dir(folder, EngineConfig(...))
+    engine.add_request("a", prompt_ids, SamplingParams(), max_new_tokens=32)
+    while engine.has_work():
+        for finished in engine.step():
+            ...
+
+Each step: plan (scheduler), run the planned tokens as one batch (runner.step),
+choose the next tokens (sampler), commit (scheduler).  The request's state
+changes only after its step has run, as in the reference's engine shell
+(v3/crates/rvllm-runtime/src/engine.rs:93-143).
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import os
+import time
+from typing import Hashable, Iterable, Optional, Sequence
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .runner import ModelRunner
+from .scheduler import Request, RequestState, Scheduler, StepPlan
+
+
+@dataclasses.dataclass
+class GenerationResult:
+    request_id: Hashable
+    prompt: list[int]
+    tokens: list[int]
+    finish_reason: str  # "stop" (an end-of-sequence id), "length", or "capacity"
+    set_backs: int = 0
+
+
+class LLMEngine:
+    def __init__(self, runner: ModelRunner):
+        self.runner = runner
+        cfg = runner.config
+        self.scheduler = Scheduler(runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.max_prefill_chunk,
+                                   cfg.max_model_len, on_admit=self._on_admit)
+        self.sampler = Sampler(runner.model.spec.vocab_size)
+        self.steps = 0
+        self.tokens_run = 0
+
+    @classmethod
+    def from_model_dir(cls, model_dir: str | os.PathLike, config: Optional[EngineConfig] = None) -> "LLMEngine":
+        return cls(ModelRunner.from_model_dir(model_dir, config or EngineConfig()))
+
+    @classmethod
+    def from_random(cls, model_config, seed: int, config: Optional[EngineConfig] = None) -> "LLMEngine":
+        return cls(ModelRunner.from_random(model_config, seed, config or EngineConfig()))
+
+    def _on_admit(self, request_id: Hashable) -> None:
+        self.runner.storage.clear_slot(self.runner.cache.slot(request_id))
+
+    # ---- requests ----------------------------------------------------
+    def add_request(self, request_id: Hashable, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+                    max_new_tokens: int = 16, eos_ids: Iterable[int] = (), ignore_eos: bool = False) -> Request:
+        vocab = self.runner.model.spec.vocab_size
+        prompt = [int(t) for t in prompt]
+        for t in prompt:
+            if not 0 <= t < vocab:
+                raise ValueError(f"token id {t} outside the vocabulary of {vocab}")
+        params = (params or SamplingParams()).validate()
+        if not params.is_greedy():
+            params.kernel_k(vocab)  # a draw over a large vocabulary needs an explicit top_k
+        req = Request(request_id, prompt, params, int(max_new_tokens), frozenset(int(e) for e in eos_ids), ignore_eos)
+        self.scheduler.add(req)
+        return req
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    # ---- one step --------------------------------------------------------
+    def step(self) -> list[GenerationResult]:
+        plan = self.scheduler.schedule()
+        results = [self._result(r) for r in plan.ended]
+        if not plan.portions:
+            return results
+        entries = []
+        wanting = []
+        for p in plan.portions:
+            tokens = p.request.tokens[p.start : p.start + p.count]
+            entries.append((p.request.id, tokens, [p.count - 1] if p.wants_token else []))
+            if p.wants_token:
+                wanting.append(p.request)
+        logits = self.runner.step(entries)
+        self.steps += 1
+        self.tokens_run += plan.num_tokens
+        chosen = self.sampler.sample(logits, [r.params for r in wanting], [r.rng for r in wanting])
+        next_tokens = {r.id: t for r, t in zip(wanting, chosen)}
+        finished = self.scheduler.commit(plan, next_tokens)
+        return results + [self._result(r) for r in finished]
+
+    @staticmethod
+    def _result(req: Request) -> GenerationResult:
+        return GenerationResult(req.id, list(req.prompt), list(req.output), req.finish_reason or "length",
+                                req.set_backs)
+
+    # ---- whole requests ----------------------------------------------------
+    def generate(self, prompts: Sequence[Sequence[int]], params=None, max_new_tokens: int = 16,
+                 eos_ids: Iterable[int] = (), ignore_eos: bool = False) -> list[GenerationResult]:
+        """Runs all prompts to their end; results in the order of the prompts.
+        ``params`` is one SamplingParams for all, or one per prompt."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params] * len(prompts)
+        base = f"gen{id(prompts):x}-"
+        for i, (prompt, sp) in enumerate(zip(prompts, params)):
+            self.add_request(f"{base}{i}", prompt, sp, max_new_tokens, eos_ids, ignore_eos)
+        done: dict = {}
+        while self.has_work():
+            for res in self.step():
+                done[res.request_id] = res
+        return [done[f"{base}{i}"] for i in range(len(prompts))]

@@ -17,6 +17,7 @@ import json
 import mmap
 import os
 import struct
+import warnings
 from pathlib import Path
 from typing import Iterable, Optional
 
@@ -128,7 +129,9 @@ class SafetensorsFile:
             count *= d
         if count == 0:
             return torch.empty(e.shape, dtype=dtype)
-        flat = torch.frombuffer(self._map, dtype=dtype, count=count, offset=self.data_start + e.begin)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore", UserWarning)  # the mapping is read-only and nothing writes to it
+            flat = torch.frombuffer(self._map, dtype=dtype, count=count, offset=self.data_start + e.begin)
         return flat.view(e.shape)
 
     def close(self) -> None:

@@ -1,0 +1,158 @@
+"""The cache manager's books: no page lost, held twice or freed twice, under
+random orders of requests; pages behind a window come back and are used again."""
+
+import random
+
+import pytest
+
+from rvllm_amd.cache import CacheBookkeepingError, CacheManager, OutOfPages, PagePool, StateSlots
+from rvllm_amd.parts.base import KVNeed, StateNeed
+
+
+def make(window=8, page_size=4, num_pages=16, max_requests=4, extra_state=False):
+    needs = [KVNeed(2, 16, window), KVNeed(2, 16, None), KVNeed(1, 32, window)]
+    if extra_state:
+        needs.append(StateNeed((4,)))
+    return CacheManager(needs, page_size, num_pages, max_requests)
+
+
+def test_layers_group_by_need():
+    m = make(extra_state=True)
+    assert set(m.groups) == {"window8", "full"}
+    assert m.groups["window8"].layers == [0, 2] and m.groups["full"].layers == [1]
+    assert m.layer_group == ["window8", "full", "window8", None] and m.state_layers == [3]
+
+
+def test_pool_refuses_double_free_and_foreign_free():
+    pool = PagePool("g", 4)
+    pages = pool.take("a", 2)
+    assert pages == [0, 1]
+    pool.give_back("a", [0])
+    with pytest.raises(CacheBookkeepingError):
+        pool.give_back("a", [0])  # twice
+    with pytest.raises(CacheBookkeepingError):
+        pool.give_back("b", [1])  # not the owner
+    with pytest.raises(OutOfPages):
+        pool.take("b", 4)
+    assert pool.free_count == 3  # the refused request took nothing
+    assert pool.take("b", 1) == [0]  # the page just given back is used again first
+    pool.check()
+
+
+def test_window_pages_come_back_and_full_pages_stay():
+    m = make(window=8, page_size=4, num_pages=16)
+    m.add_request("r")
+    m.extend("r", 10)
+    assert m.table("r", "full") == [0, 1, 2] and m.table("r", "window8") == [0, 1, 2]
+    m.commit("r", 10)
+    # the next token is at 10 and sees 3..10: page 0 (positions 0..3) is still needed
+    assert m.table("r", "window8") == [0, 1, 2]
+    m.extend("r", 12)
+    m.commit("r", 12)
+    # next token at 12 sees 5..12: page 0 has been passed
+    assert m.table("r", "window8") == [-1, 1, 2] and m.free_pages()["window8"] == 14
+    m.extend("r", 13)
+    # the page given back is the first to be used again
+    assert m.table("r", "window8") == [-1, 1, 2, 0]
+    m.commit("r", 13)
+    assert m.table("r", "full") == [0, 1, 2, 3]
+    m.check()
+    m.release("r")
+    assert m.free_pages() == {"window8": 16, "full": 16}
+    m.check()
+
+
+def test_reference_ring_vectors_scaled_down():
+    """The reference pins which slots a sliding layer uses around the wrap of
+    its ring (v3/crates/rvllm-runtime/src/gemma4_bring_up.rs:6357-6381: with
+    window 1024 a token at 1023/1024/1025 sees at most 1024 keys).  Here the
+    same edge in pages: with window 8 and pages of 4, the first page is kept
+    while the next token's position is at most 10 and given back from 11 on."""
+    for length, kept in [(8, 0), (10, 0), (11, 1), (12, 1), (15, 2)]:
+        m = make(window=8, page_size=4)
+        assert m.groups["window8"].first_kept_page(length) == kept
+        assert m.groups["full"].first_kept_page(length) == 0
+
+
+def test_out_of_pages_takes_nothing():
+    m = make(num_pages=4, page_size=4)
+    m.add_request("a")
+    m.extend("a", 12)
+    m.add_request("b")
+    with pytest.raises(OutOfPages):
+        m.extend("b", 8)
+    assert m.table("b", "full") == [] and m.table("b", "window8") == []
+    assert not m.can_extend([("b", 8)]) and m.can_extend([("b", 4)])
+    with pytest.raises(OutOfPages):
+        m.require([("a", 16), ("b", 4)])  # together they do not fit
+    m.check()
+
+
+def test_commit_without_pages_is_caught():
+    m = make()
+    m.add_request("a")
+    with pytest.raises(CacheBookkeepingError):
+        m.commit("a", 5)
+
+
+def test_slots():
+    m = make(max_requests=2)
+    a, b = m.add_request("a"), m.add_request("b")
+    assert {a.slot, b.slot} == {0, 1}
+    with pytest.raises(OutOfPages):
+        m.add_request("c")
+    m.release("a")
+    assert m.add_request("c").slot == a.slot
+    with pytest.raises(KeyError):
+        m.add_request("c")
+    s = StateSlots(1)
+    s.take("x")
+    with pytest.raises(CacheBookkeepingError):
+        s.give_back("y", 0)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_keep_the_books(seed):
+    rng = random.Random(seed)
+    window, page_size = rng.choice([(8, 4), (5, 16), (70, 16), (3, 4)])
+    m = make(window=window, page_size=page_size, num_pages=rng.choice([6, 12, 40]), max_requests=4)
+    wname = f"window{window}"
+    live: dict[str, int] = {}
+    counter = 0
+    for _ in range(400):
+        action = rng.random()
+        if (action < 0.2 and len(live) < 4) or not live:
+            counter += 1
+            name = f"r{counter}"
+            m.add_request(name)
+            live[name] = 0
+        elif action < 0.3:
+            name = rng.choice(list(live))
+            m.release(name)
+            del live[name]
+        else:
+            name = rng.choice(list(live))
+            new_len = live[name] + rng.choice([1, 1, 1, 2, 7, 30])
+            try:
+                m.extend(name, new_len)
+            except OutOfPages:
+                m.check()
+                victim = rng.choice(list(live))
+                m.release(victim)
+                del live[victim]
+                continue
+            m.commit(name, new_len)
+            live[name] = new_len
+            # every position the next token can see has a page; nothing older is held
+            first_visible = max(0, new_len - window + 1)
+            table = m.table(name, wname)
+            for pos in range(first_visible, new_len):
+                assert table[pos // page_size] >= 0
+            for i in range(first_visible // page_size):
+                assert table[i] == -1
+            assert all(p >= 0 for p in m.table(name, "full")[: -(-new_len // page_size)])
+        m.check()
+    for name in list(live):
+        m.release(name)
+    m.check()
+    assert all(free == g.pool.num_pages for free, g in zip(m.free_pages().values(), m.groups.values()))

@@ -1,0 +1,155 @@
+"""Generation through the entry points: greedy and sampled, long decoding,
+the first tokens of a sequence, requests set back when pages run out, the
+command line."""
+
+import json
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_gemma
+import rvllm_amd
+import trace_tools as tt
+from rvllm_amd.config.engine_config import EngineConfig
+from rvllm_amd.engine.engine import LLMEngine
+from rvllm_amd.sampling.params import SamplingParams
+from rvllm_amd.sampling.sampler import SplitMix64, sample_from_candidates
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_greedy(weights, cfg, prompt, output, dtype):
+    """Every generated token is the arg-max of the plain implementation's
+    logits for the tokens before it — up to the engine's tolerance, so that a
+    near-tie cannot fail the test, and nothing else can pass it."""
+    ids = list(prompt) + list(output)
+    logits = plain_gemma.forward(weights, cfg, ids[:-1], torch.float64)
+    slack = 2 * tt.TOLERANCE[dtype] * logits.abs().max().item()
+    for i, token in enumerate(output):
+        row = logits[len(prompt) - 1 + i]
+        assert row[token] >= row.max() - slack, f"token {i} ({token}) is not the arg-max: {row[token]} < {row.max()}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_python_entry(model_dirs, plain_models, dtype):
+    """Workload of the first tiny configuration: prompts of 5, 9, 13 and 17
+    tokens, 12 greedy tokens each."""
+    weights, cfg = plain_models["A"]
+    prompts = list(tt.make_sequences(cfg["vocab"], [5, 9, 13, 17], seed=0).values())
+    outputs = rvllm_amd.generate(str(model_dirs["A"]), prompts, max_tokens=12, dtype=dtype, max_model_len=64,
+                                 max_num_seqs=4, max_num_batched_tokens=64, max_prefill_chunk=64)
+    assert [len(o) for o in outputs] == [12] * 4
+    for prompt, out in zip(prompts, outputs):
+        assert_greedy(weights, cfg, prompt, out, dtype)
+    if dtype == "float32":
+        assert outputs == [plain_gemma.greedy(weights, cfg, p, 12, torch.float64) for p in prompts]
+
+
+def test_sampled_generation_with_chunked_prompts_is_the_plain_models_stream(model_dirs, plain_models):
+    """Workload of the second tiny configuration: six requests with prompts of
+    1 to 23 tokens, prompts cut into portions of 7 beside decoding requests,
+    10 tokens each at temperature 0.8 from fixed seeds.  The same draws on the
+    plain implementation's logits give the same tokens."""
+    weights, cfg = plain_models["B"]
+    prompts = list(tt.make_sequences(cfg["vocab"], [1, 5, 9, 14, 19, 23], seed=1).values())
+    engine = LLMEngine.from_model_dir(model_dirs["B"], EngineConfig(
+        dtype="float32", max_model_len=64, max_num_seqs=4, max_num_batched_tokens=16, max_prefill_chunk=7))
+    params = [SamplingParams(0.8, 0, 1.0, seed=100 + i) for i in range(len(prompts))]
+    results = engine.generate(prompts, params, max_new_tokens=10)
+    assert engine.steps > 10  # portions and decodes shared steps
+    for i, (prompt, res) in enumerate(zip(prompts, results)):
+        rng = SplitMix64(100 + i)
+        ids = list(prompt)
+        for token in res.tokens:
+            row = plain_gemma.forward(weights, cfg, ids, torch.float64)[-1].float()
+            cands = [(v / 0.8, j) for j, v in enumerate(row.tolist())]
+            want = sample_from_candidates(cands, 0, 1.0, rng, cfg["vocab"])
+            assert token == want, f"request {i}, token {len(ids) - len(prompt)}"
+            ids.append(token)
+    # the same seeds give the same streams again, other seeds give others
+    again = engine.generate(prompts, params, max_new_tokens=10)
+    assert [r.tokens for r in again] == [r.tokens for r in results]
+    other = engine.generate(prompts, [SamplingParams(0.8, 0, 1.0, seed=7 + i) for i in range(6)], max_new_tokens=10)
+    assert [r.tokens for r in other] != [r.tokens for r in results]
+
+
+def test_top_k_one_and_top_p_zero_are_greedy(model_dirs):
+    engine = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(dtype="float32", max_model_len=64, max_num_seqs=4))
+    prompt = [[7, 8, 9, 10]]
+    greedy = engine.generate(prompt, SamplingParams(), max_new_tokens=8)[0].tokens
+    assert engine.generate(prompt, SamplingParams(0.9, 1, 1.0, 5), max_new_tokens=8)[0].tokens == greedy
+    assert engine.generate(prompt, SamplingParams(0.9, 0, 0.0, 5), max_new_tokens=8)[0].tokens == greedy
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(model_dirs, plain_models, dtype):
+    """300 tokens decoded one by one: the window passes many pages, pages of
+    the window group are given back and used again by the same request."""
+    weights, cfg = plain_models["A"]
+    engine = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(
+        dtype=dtype, max_model_len=512, max_num_seqs=1, max_cache_tokens=512))
+    prompt = [11, 22, 33]
+    res = engine.generate([prompt], None, max_new_tokens=300, ignore_eos=True)[0]
+    assert len(res.tokens) == 300 and res.finish_reason == "length"
+    assert_greedy(weights, cfg, prompt, res.tokens, dtype)
+    assert engine.runner.cache.free_pages()["window8"] == engine.runner.cache.groups["window8"].pool.num_pages
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens_of_a_sequence(model_dirs, plain_models, name):
+    weights, cfg = plain_models[name]
+    engine = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(dtype="float32", max_model_len=64, max_num_seqs=2))
+    runner = engine.runner
+    ids = [cfg["vocab"] - 1, 0, 3]
+    want = plain_gemma.forward(weights, cfg, ids, torch.float64)
+    runner.add_request("x")
+    for i, t in enumerate(ids):
+        got = runner.step([("x", [t], [0])]).cpu().numpy()
+        tt.compare(got, want[i:i + 1], "float32", f"{name} position {i}")
+    runner.release("x")
+
+
+def test_requests_set_back_when_pages_run_out_give_the_same_tokens(model_dirs):
+    prompts = list(tt.make_sequences(256, [20, 28, 24, 18], seed=5).values())
+    common = dict(dtype="float32", max_model_len=128, max_num_seqs=4, max_num_batched_tokens=64, max_prefill_chunk=16)
+    roomy = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(max_cache_tokens=1024, **common))
+    tight = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(max_cache_tokens=160, **common))
+    want = roomy.generate(prompts, None, max_new_tokens=40, ignore_eos=True)
+    got = tight.generate(prompts, None, max_new_tokens=40, ignore_eos=True)
+    assert sum(r.set_backs for r in want) == 0 and sum(r.set_backs for r in got) >= 1
+    assert [r.tokens for r in got] == [r.tokens for r in want]
+    tight.runner.cache.check()
+    assert all(free == g.pool.num_pages for free, g in zip(tight.runner.cache.free_pages().values(),
+                                                           tight.runner.cache.groups.values()))
+
+
+def test_eos_and_capacity_reasons(model_dirs):
+    engine = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(dtype="float32", max_model_len=128,
+                                                                    max_num_seqs=2, max_cache_tokens=32))
+    prompt = [5, 6, 7, 8]
+    free_run = engine.generate([prompt], None, max_new_tokens=6)[0].tokens
+    stopped = engine.generate([prompt], None, max_new_tokens=6, eos_ids=[free_run[2]])[0]
+    first = free_run.index(free_run[2])
+    assert stopped.tokens == free_run[:first + 1] and stopped.finish_reason == "stop"
+    # 32 tokens of cache: a request that wants more ends with "capacity" and keeps what it produced
+    res = engine.generate([prompt], None, max_new_tokens=100, ignore_eos=True)[0]
+    assert res.finish_reason == "capacity" and 0 < len(res.tokens) < 100
+
+
+def test_command_line(model_dirs, tmp_path):
+    prompts = tmp_path / "prompts.txt"
+    prompts.write_text("1 2 3 4\n9 8 7\n")
+    dump = tmp_path / "out.txt"
+    cmd = [sys.executable, "-m", "rvllm_amd.cli", "--model", str(model_dirs["A"]), "--dtype=float32",
+           "--max-model-len", "64", "--max-num-seqs", "2", "--prompt-file", str(prompts), "--max-tokens", "5",
+           "--dump", str(dump)]
+    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=str(tt.ROOT), timeout=300)
+    assert proc.returncode == 0, proc.stderr
+    lines = [json.loads(l) for l in proc.stdout.strip().splitlines()]
+    assert [l["completion_tokens"] for l in lines] == [5, 5] and lines[0]["finish_reason"] == "length"
+    assert dump.read_text().splitlines() == [" ".join(map(str, l["token_ids"])) for l in lines]
+    direct = rvllm_amd.generate(str(model_dirs["A"]), [[1, 2, 3, 4], [9, 8, 7]], max_tokens=5, dtype="float32",
+                                max_model_len=64, max_num_seqs=2)
+    assert direct == [l["token_ids"] for l in lines]

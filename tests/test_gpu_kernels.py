@@ -1,0 +1,319 @@
+"""Each HIP kernel alone against a plain PyTorch reference of the same
+operation, at sizes other than the engine's tiny models: widths and
+vocabularies that are no power of two, head sizes in steps of 16, odd head
+groupings, pages of every size."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_gemma as P
+from rvllm_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+def dev(t, dtype=None):
+    return t.to(device=DEV, dtype=dtype or t.dtype).contiguous()
+
+
+def test_library_is_loaded_from_the_tree():
+    assert ops.library() is not None and "librvllm_amd_" in ops.library_path()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,vocab", [(80, 301), (2560, 1000)])
+def test_embed_gather(dtype, hidden, vocab):
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn(vocab, hidden, generator=g).to(dtype)
+    ids = torch.tensor([0, vocab - 1, 5, 5, 17], dtype=torch.int32)
+    out = torch.empty(5, hidden, dtype=dtype, device=DEV)
+    ops.embed_gather(dev(table), dev(ids), math.sqrt(hidden), out)
+    want = (table.float()[ids.long()] * math.sqrt(hidden)).to(dtype)
+    assert torch.equal(out.cpu(), want)  # one multiplication in 32-bit, one rounding
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [16, 100, 2560, 5376])
+@pytest.mark.parametrize("wdtype", DTYPES)
+def test_rmsnorm(dtype, width, wdtype):
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn(7, width, generator=g) * 3).to(dtype)
+    w = (torch.randn(width, generator=g) * 0.1).to(wdtype)
+    got = ops.rmsnorm(dev(x), dev(w), 1e-5, 1.0).cpu().float()
+    want = P.rmsnorm(x.double(), w.double(), 1e-5).float()
+    assert torch.allclose(got, want, **tol(dtype))
+    # offset 0: the stored weight is the gain
+    got = ops.rmsnorm(dev(x), dev(w), 1e-5, 0.0).cpu().float()
+    want = (P.rmsnorm(x.double(), torch.zeros(width).double(), 1e-5) * w.double()).float()
+    assert torch.allclose(got, want, **tol(dtype))
+
+
+def test_rmsnorm_rows_picks_rows():
+    x = torch.randn(9, 48)
+    w = torch.randn(48) * 0.1
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    got = ops.rmsnorm(dev(x), dev(w), 1e-6, 1.0, rows=dev(rows)).cpu()
+    assert torch.allclose(got, P.rmsnorm(x[rows.long()], w, 1e-6), atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [96, 2560])
+def test_add_rmsnorm_with_and_without_the_next_norm(dtype, width):
+    g = torch.Generator().manual_seed(3)
+    branch = (torch.randn(5, width, generator=g) * 2).to(dtype)
+    res = torch.randn(5, width, generator=g).to(dtype)
+    w1 = (torch.randn(width, generator=g) * 0.1).to(dtype)
+    w2 = (torch.randn(width, generator=g) * 0.1).to(dtype)
+    want_res = res.double() + P.rmsnorm(branch.double(), w1.double(), 1e-6)
+    r = dev(res.clone())
+    assert ops.add_rmsnorm(dev(branch), dev(w1), 1e-6, 1.0, r) is None
+    assert torch.allclose(r.cpu().float(), want_res.float(), **tol(dtype))
+    r2 = dev(res.clone())
+    nxt = ops.add_rmsnorm(dev(branch), dev(w1), 1e-6, 1.0, r2, dev(w2), 1e-5, 1.0)
+    assert torch.equal(r2, r)
+    # the next norm reads the residual as stored
+    want_next = P.rmsnorm(r.cpu().double(), w2.double(), 1e-5)
+    assert torch.allclose(nxt.cpu().float(), want_next.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gated_act(dtype):
+    g = torch.Generator().manual_seed(4)
+    gu = (torch.randn(6, 2 * 173, generator=g) * 2).to(dtype)
+    got = ops.gated_act(dev(gu), "gelu_pytorch_tanh").cpu().float()
+    want = F.gelu(gu[:, :173].double(), approximate="tanh") * gu[:, 173:].double()
+    assert torch.allclose(got, want.float(), **tol(dtype))
+    got = ops.gated_act(dev(gu), "silu").cpu().float()
+    want = F.silu(gu[:, :173].double()) * gu[:, 173:].double()
+    assert torch.allclose(got, want.float(), **tol(dtype))
+    with pytest.raises(ops.KernelError, match="unknown activation"):
+        ops.gated_act(dev(gu), "relu")
+
+
+def test_softcap():
+    x = torch.tensor([[1000.0, -1000.0, 0.3, 15.0]])
+    got = ops.softcap_(dev(x.clone()), 30.0).cpu()
+    assert torch.allclose(got, 30.0 * torch.tanh(x / 30.0), atol=1e-5) and abs(got[0, 0] - 30.0) < 0.01
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 100, 96), (65, 130, 257), (8, 509, 96), (200, 64, 2560)])
+def test_gemm_plain_is_true_32_bit_and_independent_of_rows(m, n, k):
+    g = torch.Generator().manual_seed(5)
+    a, w = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g)
+    out = torch.empty(m, n, device=DEV)
+    ops.gemm_plain(dev(a), dev(w), out)
+    want = (a.double() @ w.double().T)
+    # 32-bit products and sums: the error is that of a chain of k roundings, far below any 16-bit mode
+    assert (out.cpu().double() - want).abs().max() <= 1e-6 * math.sqrt(k) * want.abs().max()
+    # a row's result does not depend on the rows around it
+    one = torch.empty(1, n, device=DEV)
+    ops.gemm_plain(dev(a[m - 1:m]), dev(w), one)
+    assert torch.equal(one[0], out[m - 1])
+
+
+def test_gemm_plain_bf16_inputs_give_32_bit_logits():
+    g = torch.Generator().manual_seed(6)
+    a, w = torch.randn(5, 80, generator=g).bfloat16(), torch.randn(301, 80, generator=g).bfloat16()
+    out = torch.empty(5, 301, device=DEV, dtype=torch.float32)
+    ops.gemm_plain(dev(a), dev(w), out)
+    assert torch.allclose(out.cpu(), a.float() @ w.float().T, atol=1e-4, rtol=1e-5)
+
+
+def paged_setup(T_total, nkv, hd, page_size, dtype, seed, scramble=True):
+    """A cache whose pages are handed out in a scrambled order."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages = -(-T_total // page_size) + 3
+    order = torch.randperm(n_pages, generator=g).tolist() if scramble else list(range(n_pages))
+    k_pages = torch.zeros(n_pages, page_size, nkv, hd, dtype=dtype)
+    v_pages = torch.zeros_like(k_pages)
+    table = torch.full((1, n_pages), -1, dtype=torch.int32)
+    for i in range(-(-T_total // page_size)):
+        table[0, i] = order[i]
+    return g, k_pages, v_pages, table
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,hd,rot", [(4, 2, 16, 16), (6, 3, 48, 48), (5, 1, 80, 40), (8, 4, 256, 256), (3, 3, 128, 0)])
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size):
+    T = 37
+    g, k_pages, v_pages, table = paged_setup(T + 100, nkv, hd, page_size, dtype, 7)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd, generator=g).to(dtype)
+    qw = (torch.randn(hd, generator=g) * 0.1).to(dtype)
+    kw = (torch.randn(hd, generator=g) * 0.1).to(dtype)
+    positions = torch.arange(90, 90 + T, dtype=torch.int32)  # straddles page edges
+    inv_freq = (10000.0 ** (-2.0 * torch.arange(rot // 2, dtype=torch.float64) / hd) / 4.0).float()
+    q_out = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
+    kp, vp = dev(k_pages), dev(v_pages)
+    ops.qk_norm_rope_kv_write(dev(qkv), q_out, dev(qw), dev(kw), 1e-6, 1.0, dev(inv_freq) if rot else None, rot,
+                              dev(positions), dev(torch.zeros(T, dtype=torch.int32)), dev(table), kp, vp, nq, nkv, hd)
+    q, k, v = qkv.double().split([nq * hd, nkv * hd, nkv * hd], dim=1)
+    q = P.rmsnorm(q.view(T, nq, hd), qw.double(), 1e-6)
+    k = P.rmsnorm(k.view(T, nkv, hd), kw.double(), 1e-6)
+    if rot:
+        full = torch.zeros(hd // 2, dtype=torch.float64)  # dimensions past rot/2 get angle 0: they pass through
+        full[: rot // 2] = inv_freq.double()
+        q, k = P.rope(q, positions, full), P.rope(k, positions, full)
+    assert torch.allclose(q_out.cpu().float().view(T, nq, hd), q.float(), **tol(dtype))
+    for t in range(T):
+        pos = int(positions[t])
+        page, off = int(table[0, pos // page_size]), pos % page_size
+        assert torch.allclose(kp[page, off].cpu().float(), k[t].float(), **tol(dtype)), t
+        assert torch.equal(vp[page, off].cpu(), v[t].view(nkv, hd).to(dtype)), t  # values are stored as projected
+    # nothing else was written
+    written = {(int(table[0, int(p) // page_size]), int(p) % page_size) for p in positions}
+    mask = torch.ones(kp.shape[:2], dtype=torch.bool)
+    for page, off in written:
+        mask[page, off] = False
+    assert kp.cpu()[mask].abs().sum() == 0 and vp.cpu()[mask].abs().sum() == 0
+
+
+def test_qk_norm_rope_without_cache_write_leaves_the_cache_alone():
+    nq, nkv, hd, T = 2, 1, 32, 5
+    g, k_pages, v_pages, table = paged_setup(64, nkv, hd, 16, torch.float32, 8)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd, generator=g)
+    q_out = torch.empty(T, nq * hd, device=DEV)
+    kp, vp = dev(k_pages), dev(v_pages)
+    ops.qk_norm_rope_kv_write(dev(qkv), q_out, None, None, 0.0, 0.0, None, 0, dev(torch.arange(T, dtype=torch.int32)),
+                              dev(torch.zeros(T, dtype=torch.int32)), dev(table), kp, vp, nq, nkv, hd, write_kv=False)
+    assert kp.abs().sum() == 0 and vp.abs().sum() == 0
+    assert torch.equal(q_out.cpu(), qkv[:, : nq * hd])  # no norm, no rotation: queries pass through
+
+
+def reference_attention(q, k_all, v_all, positions, scale, window):
+    """Attention of the query tokens (at ``positions``) over keys 0..p of one request."""
+    out = torch.empty_like(q)
+    T, nq, hd = q.shape
+    group = nq // k_all.shape[1]
+    for t in range(T):
+        p = int(positions[t])
+        lo = max(0, p - window + 1) if window else 0
+        for h in range(nq):
+            s = scale * (k_all[lo:p + 1, h // group] @ q[t, h])
+            out[t, h] = torch.softmax(s, dim=0) @ v_all[lo:p + 1, h // group]
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,hd", [(4, 2, 16), (6, 1, 48), (3, 3, 80), (8, 4, 256), (2, 1, 128)])
+@pytest.mark.parametrize("window", [None, 7, 100])
+def test_paged_attention_generic(dtype, nq, nkv, hd, window):
+    ctx, page_size = 203, 16
+    g, k_pages, v_pages, table = paged_setup(ctx, nkv, hd, page_size, dtype, 9)
+    k_all = torch.randn(ctx, nkv, hd, generator=g).to(dtype)
+    v_all = torch.randn(ctx, nkv, hd, generator=g).to(dtype)
+    for j in range(ctx):
+        page, off = int(table[0, j // page_size]), j % page_size
+        k_pages[page, off], v_pages[page, off] = k_all[j], v_all[j]
+    # pages behind the window are gone: a kernel that touches them fails loudly
+    if window:
+        first_needed = max(0, 150 - window + 1) // page_size
+        for i in range(first_needed):
+            k_pages[int(table[0, i])] = float("nan")
+            table[0, i] = -1
+    positions = torch.tensor([150, 151, 160, 175, 176, 191, 192, 202], dtype=torch.int32)
+    q = torch.randn(len(positions), nq, hd, generator=g).to(dtype)
+    out = torch.empty(len(positions), nq * hd, dtype=dtype, device=DEV)
+    ops.paged_attention_generic(dev(q.view(len(positions), -1)), dev(k_pages), dev(v_pages), dev(table),
+                                dev(positions), dev(torch.zeros(len(positions), dtype=torch.int32)), out, nq,
+                                hd ** -0.5, window)
+    want = reference_attention(q.double(), k_all.double(), v_all.double(), positions, hd ** -0.5, window)
+    assert torch.allclose(out.cpu().float().view_as(want), want.float(), **tol(dtype))
+
+
+def test_paged_attention_finds_one_far_key_among_hundreds():
+    """Random keys hide a wrong mask or table; here one far key carries all
+    the weight, so the output is its value exactly."""
+    nq, nkv, hd, ctx, page_size = 2, 1, 32, 700, 16
+    g, k_pages, v_pages, table = paged_setup(ctx, nkv, hd, page_size, torch.float32, 10)
+    k_all = torch.randn(ctx, nkv, hd, generator=g) * 0.01
+    v_all = torch.randn(ctx, nkv, hd, generator=g)
+    far = 17  # on the second page
+    k_all[far, 0] = 0
+    k_all[far, 0, 3] = 40.0
+    for j in range(ctx):
+        k_pages[int(table[0, j // page_size]), j % page_size] = k_all[j]
+        v_pages[int(table[0, j // page_size]), j % page_size] = v_all[j]
+    q = torch.zeros(1, nq, hd)
+    q[0, :, 3] = 40.0
+    out = torch.empty(1, nq * hd, device=DEV)
+    args = (dev(q.view(1, -1)), dev(k_pages), dev(v_pages), dev(table), dev(torch.tensor([ctx - 1], dtype=torch.int32)),
+            dev(torch.zeros(1, dtype=torch.int32)), out, nq, 1.0)
+    ops.paged_attention_generic(*args, None)
+    assert torch.allclose(out.cpu().view(nq, hd), v_all[far, 0].expand(nq, hd), atol=1e-5)
+    # exactly at the window's edge the key is still seen, one further it is not
+    ops.paged_attention_generic(*args, ctx - far)
+    assert torch.allclose(out.cpu().view(nq, hd), v_all[far, 0].expand(nq, hd), atol=1e-5)
+    ops.paged_attention_generic(*args, ctx - far - 1)
+    assert not torch.allclose(out.cpu().view(nq, hd), v_all[far, 0].expand(nq, hd), atol=1e-2)
+
+
+def test_paged_attention_missing_page_shows():
+    nq, nkv, hd = 1, 1, 16
+    g, k_pages, v_pages, table = paged_setup(40, nkv, hd, 16, torch.float32, 11)
+    table[0, 1] = -1  # a visible page is missing: the result must not look valid
+    q = torch.randn(1, hd, generator=g)
+    out = torch.empty(1, hd, device=DEV)
+    ops.paged_attention_generic(dev(q), dev(k_pages), dev(v_pages), dev(table), dev(torch.tensor([39], dtype=torch.int32)),
+                                dev(torch.zeros(1, dtype=torch.int32)), out, nq, 1.0, None)
+    assert torch.isnan(out).all()
+
+
+@pytest.mark.parametrize("vocab", [5, 256, 509, 4097, 262208])
+def test_argmax(vocab):
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(3, vocab, generator=g)
+    x[1, vocab // 2] = x[1, vocab - 1] = 50.0  # two equal maxima: the lowest id wins
+    x[2, :] = 1.5  # all equal: id 0
+    x[0, 0] = float("nan")  # NaN is skipped
+    got = ops.argmax(dev(x)).cpu().tolist()
+    assert got == [int(torch.nan_to_num(x[0], nan=-1e9).argmax()), vocab // 2, 0]
+
+
+def test_argmax_golden_rows_of_the_reference():
+    # v3/crates/rvllm-invariants/tests/identity.rs:91-128
+    assert ops.argmax(dev(torch.tensor([[2.0, 9.0, 4.0, 9.0, 1.0]]))).item() == 1
+    assert ops.argmax(dev(torch.tensor([[1.5, 1.5, 1.5, 1.5]]))).item() == 0
+    assert ops.argmax(dev(torch.tensor([[0.1, 0.2, 9.9, 0.3], [7.0, 0.0, 1.0, 2.0]]))).cpu().tolist() == [2, 0]
+
+
+@pytest.mark.parametrize("vocab,k", [(509, 509), (300, 1), (4097, 50), (262208, 1024)])
+def test_topk_select(vocab, k):
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(2, vocab, generator=g)
+    x[1, : vocab // 2] = 0.25  # many equal values: the lower ids are taken first
+    inv_t = torch.tensor([1.0 / 0.8, 2.0])
+    vals, idx = ops.topk_select(dev(x), k, dev(inv_t))
+    vals, idx = vals.cpu(), idx.cpu().long()
+    for r in range(2):
+        order = sorted(range(vocab), key=lambda i: (-x[r, i].item(), i))[:k]
+        assert sorted(idx[r].tolist()) == sorted(order)
+        assert torch.equal(vals[r], x[r][idx[r]] * inv_t[r])
+
+
+def test_kernels_refuse_what_they_cannot_do():
+    x = torch.randn(4, 32)
+    with pytest.raises(ops.KernelError, match="GPU"):
+        ops.rmsnorm(x, torch.zeros(32), 1e-6, 1.0)
+    with pytest.raises(ops.KernelError, match="weight"):
+        ops.rmsnorm(dev(x), dev(torch.zeros(31)), 1e-6, 1.0)
+    with pytest.raises(ops.KernelError, match="dtype"):
+        ops.rmsnorm(dev(x.half()), dev(torch.zeros(32)), 1e-6, 1.0)
+    with pytest.raises(ops.KernelError, match="inner sizes"):
+        ops.gemm_plain(dev(x), dev(torch.randn(8, 31)), torch.empty(4, 8, device=DEV))
+    with pytest.raises(ops.KernelError, match="head_dim"):
+        hd = 1024
+        ops.qk_norm_rope_kv_write(dev(torch.randn(1, 3 * hd)), torch.empty(1, hd, device=DEV), None, None, 0.0, 0.0,
+                                  None, 0, dev(torch.zeros(1, dtype=torch.int32)), dev(torch.zeros(1, dtype=torch.int32)),
+                                  None, None, None, 1, 1, hd, write_kv=False)
+    with pytest.raises(ops.KernelError, match="k="):
+        ops.topk_select(dev(torch.randn(1, 5000)), 2000, dev(torch.ones(1)))

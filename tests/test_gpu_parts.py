@@ -1,0 +1,296 @@
+"""Each part of a layer alone against the plain implementation, and a toy
+mixer with a state of its own — defined here, not in the framework — that is
+registered, built from a model folder and stepped through the same engine."""
+
+import dataclasses
+import json
+import math
+
+import pytest
+import torch
+
+import plain_gemma as P
+from rvllm_amd.cache.manager import CacheManager
+from rvllm_amd.cache.storage import CacheStorage
+from rvllm_amd.config.engine_config import EngineConfig
+from rvllm_amd.engine.batch import BatchBuilder, Portion
+from rvllm_amd.engine.runner import ModelRunner
+from rvllm_amd.models import Architecture, register_architecture, unregister_architecture
+from rvllm_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, LayerSpec, Mixer, ModelSpec,
+                             ParamSpec, PartSpec, ScheduleEntry, StateNeed)
+from rvllm_amd.weights.random_init import random_tensors, write_random_model
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def bound(part, prefix, dtype, seed=0):
+    tensors = random_tensors(part.param_specs(prefix), seed, "cpu", dtype)
+    part.bind(tensors, prefix, DEV, dtype)
+    return {k: v.double() for k, v in tensors.items()}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    norm = NORMS.build(PartSpec("rmsnorm", {"eps": 1e-5, "unit_offset": True}), width=72, name="some_norm")
+    assert [s.name for s in norm.param_specs("model.layers.3")] == ["model.layers.3.some_norm.weight"]
+    w = bound(norm, "model.layers.3", dtype)["model.layers.3.some_norm.weight"]
+    x = torch.randn(5, 72).to(dtype)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(norm.forward(x.to(DEV)).cpu().double(), P.rmsnorm(x.double(), w, 1e-5), atol=tol, rtol=tol)
+    plain = NORMS.build(PartSpec("rmsnorm", {"eps": 1e-5}), width=72, name="n")
+    plain.bind({"p.n.weight": w.to(dtype)}, "p", DEV, dtype)
+    want = P.rmsnorm(x.double(), torch.zeros(72).double(), 1e-5) * w.to(dtype).double()
+    assert torch.allclose(plain.forward(x.to(DEV)).cpu().double(), want, atol=tol, rtol=tol)
+
+
+def test_rope_part_tables():
+    rope = POSITION_ENCODINGS.build(PartSpec("rope", {"theta": 5e5, "factor": 4.0}), head_dim=32)
+    assert rope.rotary_dim == 32
+    assert torch.equal(rope.inv_freq(DEV).cpu(), P.rope_inv_freq(32, 5e5, 4.0))
+    none = POSITION_ENCODINGS.build(PartSpec("none"), head_dim=32)
+    assert none.rotary_dim == 0 and none.inv_freq(DEV) is None
+    with pytest.raises(ValueError):
+        POSITION_ENCODINGS.build(PartSpec("rope", {"theta": 1e4, "rotary_dim": 7}), head_dim=32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    ff = FEED_FORWARDS.build(PartSpec("gated_mlp", {"intermediate_size": 88, "activation": "gelu_pytorch_tanh"}),
+                             hidden_size=40)
+    w = bound(ff, "L", dtype)
+    x = torch.randn(6, 40).to(dtype)
+    want = P.feed_forward(x.double(), w["L.mlp.gate_proj.weight"], w["L.mlp.up_proj.weight"],
+                          w["L.mlp.down_proj.weight"])
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    got = ff.forward(x.to(DEV), None).cpu().double()
+    assert (got - want).abs().max() <= tol * max(1.0, want.abs().max().item())
+
+
+def attention_harness(mixer, page_size=16, num_pages=32, max_tokens=256):
+    cache = CacheManager([mixer.cache_need()], page_size, num_pages, 2)
+    storage = CacheStorage(cache, DEV, mixer.w_o.dtype)
+    builder = BatchBuilder(DEV, max_tokens, 2, {name: num_pages for name in cache.groups})
+    return cache, storage, builder
+
+
+def run_portions(mixer, x, cuts):
+    """Feed x[T, H] of one request through the mixer in portions."""
+    cache, storage, builder = attention_harness(mixer)
+    cache.add_request("r")
+    outs, start = [], 0
+    group = next(iter(cache.groups))
+    for n in cuts:
+        cache.extend("r", start + n)
+        batch = builder.build([Portion("r", [0] * n, start)], {group: [cache.table("r", group)]}, [cache.slot("r")])
+        outs.append(mixer.forward(x[start:start + n].to(DEV), batch, storage.views[0]).cpu())
+        cache.commit("r", start + n)
+        start += n
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window,rope", [(None, True), (6, True), (None, False), (20, False)])
+def test_attention_part(dtype, window, rope):
+    H, nq, nkv, hd, T = 56, 6, 2, 16, 45
+    spec = PartSpec("attention", {
+        "num_heads": nq, "num_kv_heads": nkv, "head_dim": hd, "scale": 0.2, "window": window,
+        "qk_norm": {"eps": 1e-6, "unit_offset": True},
+        "position": PartSpec("rope", {"theta": 1e4, "factor": 2.0}) if rope else PartSpec("none"),
+    })
+    mixer = MIXERS.build(spec, hidden_size=H)
+    w = bound(mixer, "L", dtype, seed=3)
+    x = torch.randn(T, H).to(dtype)
+    # the plain layer's attention branch
+    xd = x.double()
+    q = P.rmsnorm((xd @ w["L.self_attn.q_proj.weight"].T).view(T, nq, hd), w["L.self_attn.q_norm.weight"], 1e-6)
+    k = P.rmsnorm((xd @ w["L.self_attn.k_proj.weight"].T).view(T, nkv, hd), w["L.self_attn.k_norm.weight"], 1e-6)
+    v = (xd @ w["L.self_attn.v_proj.weight"].T).view(T, nkv, hd)
+    if rope:
+        inv = P.rope_inv_freq(hd, 1e4, 2.0, torch.float64)
+        q, k = P.rope(q, torch.arange(T), inv), P.rope(k, torch.arange(T), inv)
+    want = P.attention(q, k, v, 0.2, window).reshape(T, nq * hd) @ w["L.self_attn.o_proj.weight"].T
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    for cuts in ([T], [17, 1, 1, 2, 16, 8]):
+        got = run_portions(mixer, x, cuts).double()
+        assert (got - want).abs().max() <= tol * max(1.0, want.abs().max().item()), cuts
+
+
+def test_attention_without_rotation_or_norm_is_plain_softmax_attention():
+    """The special case that reduces to the library routine."""
+    H, nq, hd, T = 32, 2, 16, 12
+    spec = PartSpec("attention", {"num_heads": nq, "num_kv_heads": nq, "head_dim": hd, "scale": hd ** -0.5,
+                                  "window": None, "qk_norm": None, "position": None})
+    mixer = MIXERS.build(spec, hidden_size=H)
+    assert len(mixer.param_specs("L")) == 4  # no norm weights asked for
+    w = bound(mixer, "L", torch.float32, seed=4)
+    x = torch.randn(T, H)
+    q, k, v = ((x.double() @ w[f"L.self_attn.{n}_proj.weight"].T).view(T, nq, hd).transpose(0, 1) for n in "qkv")
+    lib = torch.nn.functional.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+    want = lib.transpose(0, 1).reshape(T, nq * hd) @ w["L.self_attn.o_proj.weight"].T
+    assert torch.allclose(run_portions(mixer, x, [5, 7]).double(), want, atol=1e-5)
+
+
+def test_block_part_is_the_plain_layer(plain_models):
+    from rvllm_amd.models.gemma3 import build_spec
+    from rvllm_amd.config.gemma3 import Gemma3Config
+    import tiny_models
+
+    weights, cfg = plain_models["B"]
+    spec = build_spec(Gemma3Config.from_dict(tiny_models.CONFIG_B))
+    for layer_index in (0, 2):  # a sliding and a global layer
+        layer = spec.layers[layer_index]
+        block = BLOCKS.build(layer.block, layer=layer, hidden_size=spec.hidden_size)
+        block.bind({k: v.float() for k, v in weights.items()}, layer.prefix, DEV, torch.float32)
+        T = 19
+        x = torch.randn(T, spec.hidden_size)
+        want = P.layer(x.double(), torch.arange(T), {k: v.double() for k, v in weights.items()}, layer.prefix, cfg,
+                       cfg["kinds"][layer_index])
+        cache, storage, builder = attention_harness(block.mixer)
+        cache.add_request("r")
+        cache.extend("r", T)
+        group = next(iter(cache.groups))
+        batch = builder.build([Portion("r", [0] * T, 0)], {group: [cache.table("r", group)]}, [0])
+        xs = x.to(DEV)
+        assert block.forward(xs, batch, storage.views[0]) is None  # no next norm was asked for
+        assert torch.allclose(xs.cpu().double(), want, atol=2e-5)
+
+
+# --------------------------------------------------------------------------
+# A toy mixer with a state of its own, and a toy architecture around it.
+# --------------------------------------------------------------------------
+class RunningMeanMixer(Mixer):
+    """y[t] = W @ mean(x[0..t]): keeps the running sum and the count of a
+    request in a slot of fixed size, portions must continue where the slot
+    left off."""
+
+    def __init__(self, spec, *, hidden_size):
+        self.hidden = hidden_size
+        self.w = None
+
+    def param_specs(self, prefix):
+        return [ParamSpec(f"{prefix}.mean_mixer.weight", (self.hidden, self.hidden), init=("normal", 0.3))]
+
+    def bind(self, tensors, prefix, device, dtype):
+        self.w = tensors[f"{prefix}.mean_mixer.weight"].to(device=device, dtype=dtype)
+
+    def cache_need(self):
+        return StateNeed((self.hidden + 1,), torch.float32)
+
+    def forward(self, x, step, cache):
+        out = torch.empty_like(x)
+        starts = step.host_q_start
+        slots = step.state_slot.cpu().tolist()
+        for b in range(step.num_requests):
+            lo, hi = int(starts[b]), int(starts[b + 1])
+            state = cache.slots[slots[b]]
+            sums = state[: self.hidden] + torch.cumsum(x[lo:hi].float(), dim=0)
+            counts = state[self.hidden] + torch.arange(1, hi - lo + 1, device=x.device, dtype=torch.float32)
+            out[lo:hi] = ((sums / counts[:, None]).to(x.dtype) @ self.w.T)
+            if cache.writes:
+                state[: self.hidden] = sums[-1]
+                state[self.hidden] = counts[-1]
+        return out
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyConfig:
+    architecture: str
+    hidden: int
+    vocab: int
+    layers: int
+
+    @classmethod
+    def from_dict(cls, doc, source="config.json"):
+        return cls(doc["architectures"][0], doc["toy_hidden"], doc["toy_vocab"], doc["toy_layers"])
+
+    def to_dict(self):
+        return {"architectures": [self.architecture], "toy_hidden": self.hidden, "toy_vocab": self.vocab,
+                "toy_layers": self.layers}
+
+
+def toy_spec(cfg: ToyConfig, prefix="model") -> ModelSpec:
+    norm = PartSpec("rmsnorm", {"eps": 1e-6, "unit_offset": False})
+    attn = PartSpec("attention", {"num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "scale": 0.25, "window": None,
+                                  "qk_norm": None, "position": PartSpec("rope", {"theta": 100.0})})
+    ff = PartSpec("gated_mlp", {"intermediate_size": 2 * cfg.hidden, "activation": "silu"})
+    layers = []
+    for l in range(cfg.layers):
+        mixer = PartSpec("running_mean") if l % 2 == 0 else attn  # different mixers in different layers
+        layers.append(LayerSpec(f"{prefix}.layers.{l}", PartSpec("sandwich"), mixer, ff, norm))
+    # the order of layers is data: layer 1 runs twice, the second time reading its own cache only
+    schedule = [ScheduleEntry(l) for l in range(cfg.layers)] + [ScheduleEntry(1, cache_from=1)]
+    return ModelSpec(cfg.architecture, cfg.hidden, cfg.vocab, 512, PartSpec("scaled_embedding", {"scale": 1.0}),
+                     tuple(layers), tuple(schedule), norm, PartSpec("lm_head", {"tied": True}), prefix)
+
+
+@pytest.fixture
+def toy_architecture():
+    MIXERS.register("running_mean", RunningMeanMixer, replace=True)
+    arch = register_architecture(Architecture("ToyForCausalLM", ToyConfig.from_dict, toy_spec, ToyConfig.to_dict),
+                                 replace=True)
+    yield arch
+    unregister_architecture("ToyForCausalLM")
+    MIXERS.unregister("running_mean")
+
+
+def toy_plain(weights, cfg: ToyConfig, ids):
+    """The toy model on a whole sequence, written out plainly."""
+    w = {k: v.double() for k, v in weights.items()}
+    norm = lambda x, name: x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6) * w[name]
+    x = w["model.embed_tokens.weight"][ids]
+    T = len(ids)
+    kept = {}  # keys and values of a layer's first run; a run that reads another run's cache uses these
+    for run, l in enumerate(list(range(cfg.layers)) + [1]):
+        p = f"model.layers.{l}"
+        h = norm(x, f"{p}.input_layernorm.weight")
+        if l % 2 == 0:
+            mean = torch.cumsum(h, 0) / torch.arange(1, T + 1, dtype=torch.float64)[:, None]
+            a = mean @ w[f"{p}.mean_mixer.weight"].T
+        else:
+            inv = P.rope_inv_freq(16, 100.0, 1.0, torch.float64)
+            q = P.rope((h @ w[f"{p}.self_attn.q_proj.weight"].T).view(T, 2, 16), torch.arange(T), inv)
+            if run < cfg.layers:
+                k = P.rope((h @ w[f"{p}.self_attn.k_proj.weight"].T).view(T, 1, 16), torch.arange(T), inv)
+                kept[l] = (k, (h @ w[f"{p}.self_attn.v_proj.weight"].T).view(T, 1, 16))
+            k, v = kept[l]
+            a = P.attention(q, k, v, 0.25, None).reshape(T, 32) @ w[f"{p}.self_attn.o_proj.weight"].T
+        x = x + norm(a, f"{p}.post_attention_layernorm.weight")
+        h = norm(x, f"{p}.pre_feedforward_layernorm.weight")
+        f = (torch.nn.functional.silu(h @ w[f"{p}.mlp.gate_proj.weight"].T) * (h @ w[f"{p}.mlp.up_proj.weight"].T)) \
+            @ w[f"{p}.mlp.down_proj.weight"].T
+        x = x + norm(f, f"{p}.post_feedforward_layernorm.weight")
+    return norm(x, "model.norm.weight") @ w["model.embed_tokens.weight"].T
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, toy_architecture):
+    cfg = ToyConfig("ToyForCausalLM", hidden=24, vocab=50, layers=3)
+    folder = write_random_model(tmp_path / "toy", cfg, seed=7, dtype=torch.float32)
+    assert json.loads((folder / "config.json").read_text())["toy_hidden"] == 24
+    engine_cfg = EngineConfig(dtype="float32", max_model_len=128, max_num_seqs=3, max_num_batched_tokens=128,
+                              max_prefill_chunk=128, max_cache_tokens=256)
+    runner = ModelRunner.from_model_dir(folder, engine_cfg)
+    # layer 0 and 2 keep a state slot, layer 1 keeps pages
+    assert runner.cache.state_layers == [0, 2] and runner.cache.layer_group == [None, "full", None]
+    weights = P.load_weights(folder)
+    seqs = {"a": [3, 14, 15, 9, 26, 5, 35, 8, 9, 7, 9, 3], "b": [2, 7, 18, 28, 18, 28, 4, 5]}
+    want = {k: toy_plain(weights, cfg, v) for k, v in seqs.items()}
+    # whole
+    for name, ids in seqs.items():
+        runner.add_request(name)
+        got = runner.step([(name, ids, list(range(len(ids))))]).cpu().double()
+        assert torch.allclose(got, want[name], atol=1e-4), name
+        runner.release(name)
+    # cut and mixed: the slot carries the state from portion to portion, and a
+    # slot that is handed out again starts from zero
+    runner.add_request("a2")
+    runner.add_request("b2")
+    g1 = runner.step([("a2", seqs["a"][:5], list(range(5))), ("b2", seqs["b"][:2], [0, 1])]).cpu().double()
+    g2 = runner.step([("b2", seqs["b"][2:3], [0]), ("a2", seqs["a"][5:], list(range(7)))]).cpu().double()
+    g3 = runner.step([("b2", seqs["b"][3:], list(range(5)))]).cpu().double()
+    got_a = torch.cat([g1[:5], g2[1:]])
+    got_b = torch.cat([g1[5:], g2[:1], g3])
+    assert torch.allclose(got_a, want["a"], atol=1e-4) and torch.allclose(got_b, want["b"], atol=1e-4)
+    runner.release("a2")
+    runner.release("b2")
+    runner.cache.check()

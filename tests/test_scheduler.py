@@ -1,0 +1,209 @@
+"""The scheduler's decisions, with a step function that needs no GPU: the
+next token is a fixed function of all tokens before it, so any mistake in
+cutting, ordering, setting back or finishing changes the output."""
+
+import pytest
+
+from rvllm_amd.cache import CacheManager, OutOfPages
+from rvllm_amd.engine.scheduler import Request, RequestState, Scheduler, SchedulerError
+from rvllm_amd.parts.base import KVNeed
+from rvllm_amd.sampling.params import SamplingParams
+
+VOCAB = 97
+
+
+def next_token(tokens):
+    h = 7
+    for t in tokens:
+        h = (h * 31 + t + 1) % 1000003
+    return h % VOCAB
+
+
+def expected_output(prompt, n, eos=()):
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = next_token(seq)
+        out.append(t)
+        seq.append(t)
+        if t in eos:
+            break
+    return out
+
+
+class FakeRunner:
+    """Keeps the cache's books as the real step does and checks that every
+    request's tokens arrive once, in order."""
+
+    def __init__(self, cache):
+        self.cache = cache
+        self.seen = {}
+        self.steps = []
+
+    def step(self, plan):
+        entries = [(p.request.id, p.request.tokens[p.start:p.start + p.count], p.wants_token) for p in plan.portions]
+        self.cache.require([(rid, self.cache.length(rid) + len(toks)) for rid, toks, _ in entries])
+        out = {}
+        for rid, toks, wants in entries:
+            start = self.cache.length(rid)
+            if start == 0:
+                self.seen[rid] = []
+            assert start == len(self.seen[rid]), "tokens must continue where the cache ends"
+            self.cache.extend(rid, start + len(toks))
+            self.seen[rid] += toks
+            self.cache.commit(rid, start + len(toks))
+            if wants:
+                out[rid] = next_token(self.seen[rid])
+        self.steps.append([(rid, len(toks)) for rid, toks, _ in entries])
+        self.cache.check()
+        return out
+
+
+def build(num_pages=64, page_size=4, window=8, max_num_seqs=4, budget=16, chunk=8, max_model_len=256):
+    cache = CacheManager([KVNeed(1, 8, window), KVNeed(1, 8, None)], page_size, num_pages, max_num_seqs)
+    sched = Scheduler(cache, max_num_seqs, budget, chunk, max_model_len)
+    return sched, FakeRunner(cache)
+
+
+def run(sched, runner, limit=2000):
+    done = {}
+    for _ in range(limit):
+        if not sched.has_work():
+            break
+        plan = sched.schedule()
+        for r in plan.ended:
+            done[r.id] = r
+        if plan.portions:
+            for r in sched.commit(plan, runner.step(plan)):
+                done[r.id] = r
+    assert not sched.has_work(), "the scheduler did not finish"
+    return done
+
+
+def test_prompt_is_cut_into_portions_under_the_budget():
+    sched, runner = build(budget=16, chunk=8)
+    sched.add(Request("a", list(range(1, 21)), max_new_tokens=3))
+    done = run(sched, runner)
+    assert runner.steps[:3] == [[("a", 8)], [("a", 8)], [("a", 4)]]
+    assert runner.steps[3:] == [[("a", 1)], [("a", 1)]]  # the last token chosen is never run
+    assert done["a"].output == expected_output(range(1, 21), 3) and done["a"].finish_reason == "length"
+
+
+def test_decodes_come_first_and_prompts_fill_the_rest():
+    sched, runner = build(budget=10, chunk=8)
+    sched.add(Request("a", [1, 2, 3], max_new_tokens=6))
+    plan = sched.schedule()
+    sched.commit(plan, runner.step(plan))
+    sched.add(Request("b", list(range(1, 30)), max_new_tokens=2))
+    plan = sched.schedule()
+    # a decodes one token, b gets a portion beside it, within the budget
+    assert [(p.request.id, p.count, p.wants_token) for p in plan.portions] == [("a", 1, True), ("b", 8, False)]
+    assert plan.num_tokens <= 10
+    sched.commit(plan, runner.step(plan))
+    done = run(sched, runner)
+    assert done["a"].output == expected_output([1, 2, 3], 6)
+    assert done["b"].output == expected_output(range(1, 30), 2)
+
+
+def test_budget_is_shared_between_prompts():
+    sched, runner = build(budget=12, chunk=8)
+    sched.add(Request("a", list(range(1, 11)), max_new_tokens=1))
+    sched.add(Request("b", list(range(1, 11)), max_new_tokens=1))
+    plan = sched.schedule()
+    assert [(p.request.id, p.count) for p in plan.portions] == [("a", 8), ("b", 4)]
+
+
+def test_max_num_seqs_limits_admission():
+    sched, runner = build(max_num_seqs=2)
+    for name in "abc":
+        sched.add(Request(name, [1, 2], max_new_tokens=2))
+    plan = sched.schedule()
+    assert [p.request.id for p in plan.portions] == ["a", "b"] and len(sched.waiting) == 1
+    sched.commit(plan, runner.step(plan))
+    done = run(sched, runner)
+    assert set(done) == {"a", "b", "c"}
+
+
+def test_eos_stops_and_ignore_eos_does_not():
+    prompt = [5, 6, 7]
+    full = expected_output(prompt, 12)
+    eos = full[4]
+    first = full.index(eos)
+    sched, runner = build()
+    sched.add(Request("a", prompt, max_new_tokens=12, eos_ids=frozenset([eos])))
+    sched.add(Request("b", prompt, max_new_tokens=12, eos_ids=frozenset([eos]), ignore_eos=True))
+    done = run(sched, runner)
+    assert done["a"].output == full[:first + 1] and done["a"].finish_reason == "stop"
+    assert done["b"].output == full and done["b"].finish_reason == "length"
+
+
+def test_context_limit_bounds_new_tokens():
+    sched, runner = build(max_model_len=12)
+    sched.add(Request("a", list(range(1, 10)), max_new_tokens=50))
+    done = run(sched, runner)
+    assert len(done["a"].output) == 3  # 9 + 3 = 12 (worker.rs:1067-1080)
+    with pytest.raises(SchedulerError, match="max_model_len"):
+        sched.add(Request("b", list(range(12)), max_new_tokens=1))
+
+
+def test_bad_requests_are_refused():
+    sched, _ = build()
+    sched.add(Request("a", [1], max_new_tokens=1))
+    with pytest.raises(SchedulerError, match="duplicate"):
+        sched.add(Request("a", [1], max_new_tokens=1))
+    with pytest.raises(SchedulerError, match="empty"):
+        sched.add(Request("b", [], max_new_tokens=1))
+    with pytest.raises(SchedulerError, match="max_new_tokens"):
+        sched.add(Request("c", [1], max_new_tokens=0))
+    with pytest.raises(ValueError):
+        sched.add(Request("d", [1], SamplingParams(temperature=-1.0)))
+
+
+def test_pages_run_out_latest_request_is_set_back_and_output_is_unchanged():
+    # 10 pages of 4 tokens; three requests that need 5 + 5 + 5 pages in the full group by their end
+    prompts = {"a": list(range(1, 9)), "b": list(range(11, 19)), "c": list(range(21, 29))}
+    sched, runner = build(num_pages=10, page_size=4, budget=32, chunk=8, max_num_seqs=3)
+    for name, p in prompts.items():
+        sched.add(Request(name, p, max_new_tokens=12))
+    done = run(sched, runner)
+    for name, p in prompts.items():
+        assert done[name].output == expected_output(p, 12), name
+    assert sum(r.set_backs for r in done.values()) >= 1
+    # the oldest request is never the one set back
+    assert done["a"].set_backs == 0
+    assert runner.cache.free_pages() == {"window8": 10, "full": 10}
+
+
+def test_set_back_request_resumes_its_random_stream():
+    prompts = {"a": list(range(1, 9)), "b": list(range(11, 19))}
+    sched, runner = build(num_pages=6, page_size=4, budget=32, chunk=8, max_num_seqs=2)
+    reqs = {n: Request(n, p, SamplingParams(0.8, 10, 1.0, seed=3), max_new_tokens=10) for n, p in prompts.items()}
+    for r in reqs.values():
+        sched.add(r)
+    done = run(sched, runner)
+    assert done["b"].set_backs >= 1
+    assert reqs["b"].rng.state == 3  # the fake step draws nothing: the stream was neither reset nor replaced
+    assert done["b"].output == expected_output(prompts["b"], 10)
+
+
+def test_a_request_too_large_for_the_pool_ends_with_capacity():
+    sched, runner = build(num_pages=3, page_size=4, budget=32, chunk=8)
+    sched.add(Request("a", list(range(1, 9)), max_new_tokens=20))  # 8 + 20 tokens need 7 pages
+    sched.add(Request("b", [1, 2], max_new_tokens=2))
+    done = run(sched, runner)
+    assert done["a"].finish_reason == "capacity" and len(done["a"].output) < 20
+    assert done["a"].output == expected_output(range(1, 9), len(done["a"].output))
+    assert done["b"].output == expected_output([1, 2], 2) and done["b"].finish_reason == "length"
+    assert runner.cache.free_pages() == {"window8": 3, "full": 3}
+    small, _ = build(num_pages=1, page_size=4, chunk=8)
+    with pytest.raises(SchedulerError, match="does not fit"):
+        small.add(Request("c", list(range(1, 40)), max_new_tokens=1))  # its first portion alone needs two pages
+
+
+def test_state_changes_only_after_the_step():
+    sched, runner = build()
+    req = Request("a", [1, 2, 3], max_new_tokens=2)
+    sched.add(req)
+    plan = sched.schedule()
+    assert req.state is RequestState.RUNNING and req.computed == 0 and req.output == []
+    sched.commit(plan, runner.step(plan))
+    assert req.computed == 3 and len(req.output) == 1
