@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at Gemma-3-4B layer sizes.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
+
+Default run: the layer sizes of the 4B-sized configuration (34 layers, 5
+sliding : 1 global, hidden 2560, 8 query / 4 key-value heads of 256, GeGLU
+10240, vocabulary 262 208), random weights N(0, 0.02), bf16, 8 requests with
+8 192 tokens of context each.  One "step" is one decode step of the whole
+batch through the engine's own step function and sampler (greedy): every
+request gets one new token.  The caches are filled with random keys and values
+for the contexts (a decode step's work does not depend on their values); the
+prefill figure is measured on a real prompt of 2 048 tokens run through the
+same step function.
+
+One JSON line goes to standard output.  ``value`` is decoded tokens a second.
+``roofline`` prices the decode step against 8 TB/s: the bytes it must read
+(every weight it uses once, and the keys and values of the live requests that
+a token may see) over its time.  ``prefill.frac`` prices the prompt's flops
+against 2.5 PFLOP/s (dense bf16 MFMA).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+GEMMA3_4B = {
+    "architectures": ["Gemma3ForCausalLM"],
+    "num_hidden_layers": 34,
+    "sliding_window_pattern": 6,
+    "hidden_size": 2560,
+    "num_attention_heads": 8,
+    "num_key_value_heads": 4,
+    "head_dim": 256,
+    "intermediate_size": 10240,
+    "vocab_size": 262208,
+    "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 131072,
+    "sliding_window": 1024,
+    "rope_theta": 1000000.0,
+    "rope_local_base_freq": 10000.0,
+    "rope_scaling": {"rope_type": "linear", "factor": 8.0},
+    "query_pre_attn_scalar": 256,
+    "hidden_activation": "gelu_pytorch_tanh",
+    "tie_word_embeddings": True,
+    "final_logit_softcapping": None,
+}
+FULL_LAYERS = GEMMA3_4B["num_hidden_layers"]
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def model_numbers(cfg, elem_bytes: int):
+    """Bytes of the weights a step reads, and flops per token of the matrix products."""
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    per_layer = (cfg.q_size + 2 * cfg.kv_size) * H + H * cfg.q_size + 3 * H * I
+    norms = 4 * H + 2 * cfg.head_dim
+    layer_params = cfg.num_hidden_layers * (per_layer + norms) + H
+    weight_bytes = (layer_params + V * H) * elem_bytes  # the head reads the (tied) table once
+    return weight_bytes, 2 * cfg.num_hidden_layers * per_layer, 2 * V * H
+
+
+def kv_bytes_per_request(cfg, context: int, elem_bytes: int) -> int:
+    per_token = 2 * cfg.kv_size * elem_bytes
+    total = 0
+    for l in range(cfg.num_hidden_layers):
+        seen = min(context, cfg.sliding_window) if cfg.is_sliding(l) else context
+        total += seen * per_token
+    return total
+
+
+def attention_flops(cfg, start: int, count: int) -> int:
+    """Flops of QK^T and PV for tokens start .. start+count-1 of one request."""
+    total = 0
+    for l in range(cfg.num_hidden_layers):
+        w = cfg.sliding_window if cfg.is_sliding(l) else None
+        # sum over positions p of the number of visible keys
+        if w is None:
+            keys = sum(range(start + 1, start + count + 1))
+        else:
+            keys = sum(min(p + 1, w) for p in range(start, start + count))
+        total += 4 * cfg.num_attention_heads * cfg.head_dim * keys
+    return total
+
+
+def fill_cache(runner, batch: int, context: int, torch):
+    """Live requests with ``context`` tokens each, their pages filled with random keys and values."""
+    ids = []
+    for b in range(batch):
+        rid = f"bench-{b}"
+        runner.add_request(rid)
+        runner.cache.adopt_length(rid, context)
+        ids.append(rid)
+    gen = torch.Generator(device=runner.device)
+    gen.manual_seed(1)
+    for view in runner.storage.views:
+        if view is not None and hasattr(view, "k_pages"):
+            view.k_pages.normal_(0.0, 1.0, generator=gen)
+            view.v_pages.normal_(0.0, 1.0, generator=gen)
+    return ids
+
+
+def release_all(runner, ids):
+    for rid in ids:
+        runner.release(rid)
+
+
+def time_decode(engine_parts, batch: int, context: int, steps: int, warmup: int):
+    torch, runner, sampler, SamplingParams, SplitMix64 = engine_parts
+    ids = fill_cache(runner, batch, context - 1, torch)
+    params = [SamplingParams() for _ in ids]
+    rngs = [SplitMix64(0) for _ in ids]
+    tokens = [(17 * b + 5) % runner.model.spec.vocab_size for b in range(batch)]
+
+    def one_step(tokens):
+        logits = runner.step([(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
+        return sampler.sample(logits, params, rngs)  # greedy: arg-max on the device, ids back on the host
+
+    for _ in range(warmup):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    release_all(runner, ids)
+    return elapsed / steps
+
+
+def time_prefill(engine_parts, length: int, repeats: int):
+    torch, runner, sampler, SamplingParams, SplitMix64 = engine_parts
+    vocab = runner.model.spec.vocab_size
+    g = torch.Generator().manual_seed(2)
+    prompt = torch.randint(0, vocab, (length,), generator=g).tolist()
+    best = None
+    for i in range(repeats + 1):
+        rid = f"prefill-{i}"
+        runner.add_request(rid)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = runner.step([(rid, prompt, [length - 1])])
+        sampler.sample(logits, [SamplingParams()], [SplitMix64(0)])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        runner.release(rid)
+        if i > 0:  # the first run warms up
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers of the same size (named in config)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--graphs", type=int, default=1, help="replay decode steps from captured HIP graphs (0 = off)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
+        return 2
+
+    import torch
+
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.config.gemma3 import Gemma3Config
+    from rvllm_amd.engine.runner import ModelRunner
+    from rvllm_amd.sampling.params import SamplingParams
+    from rvllm_amd.sampling.sampler import Sampler, SplitMix64
+    import rvllm_amd.models  # noqa: F401
+
+    doc = dict(GEMMA3_4B, num_hidden_layers=args.layers)
+    cfg = Gemma3Config.from_dict(doc, "bench configuration")
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    elem = 2 if short == "bf16" else 4
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    steps_total = args.steps + args.warmup + 8
+    engine_cfg = EngineConfig(
+        dtype=args.dtype, page_size=16, max_model_len=args.context + steps_total,
+        max_num_seqs=max_batch, max_num_batched_tokens=max(args.prefill_tokens, max_batch),
+        max_prefill_chunk=max(args.prefill_tokens, 1), max_cache_tokens=max_batch * (args.context + steps_total + 16),
+        use_graphs=bool(args.graphs))
+    log(f"building {args.layers}-layer model with random weights ({short})")
+    t0 = time.time()
+    runner = ModelRunner.from_random(cfg, 0, engine_cfg)
+    torch.cuda.synchronize()
+    log(f"model ready in {time.time() - t0:.1f} s; cache {runner.storage.bytes / 2**30:.1f} GiB")
+    parts = (torch, runner, Sampler(cfg.vocab_size), SamplingParams, SplitMix64)
+
+    weight_bytes, layer_flops_per_token, head_flops_per_row = model_numbers(cfg, elem)
+
+    def decode_point(batch, steps, warmup):
+        sec = time_decode(parts, batch, args.context, steps, warmup)
+        log(f"decode batch {batch}: {sec * 1e3:.3f} ms/step, {batch / sec:.1f} tok/s")
+        return sec
+
+    sec = decode_point(args.batch, args.steps, args.warmup)
+    value = args.batch / sec
+    step_bytes = weight_bytes + args.batch * kv_bytes_per_request(cfg, args.context, elem)
+    achieved = step_bytes / sec / 1e9
+    result = {
+        "metric": "decode tok/s at batch 8, context 8192 (Gemma-3-4B sizes)",
+        "value": round(value, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": short,
+        "data": "synthetic: random weights N(0,0.02), caches filled with random keys and values, uniform token ids",
+        "config": {
+            "model": "gemma3-4b-sized dense decoder",
+            "global_batch": args.batch,
+            "seq_len": args.context,
+            "parallelism": "single GPU",
+            "layers": args.layers,
+            "layers_of_named_config": FULL_LAYERS,
+            "hidden_size": cfg.hidden_size,
+            "num_attention_heads": cfg.num_attention_heads,
+            "num_key_value_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim,
+            "intermediate_size": cfg.intermediate_size,
+            "vocab_size": cfg.vocab_size,
+            "sliding_window": cfg.sliding_window,
+            "sliding_to_global": "5:1",
+            "rope_local_global_factor": "1e4/1e6/8",
+            "page_size": engine_cfg.page_size,
+            "hip_graphs": bool(args.graphs),
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+    }
+    if not args.no_prefill:
+        T = args.prefill_tokens
+        psec = time_prefill(parts, T, repeats=2)
+        flops = T * layer_flops_per_token + attention_flops(cfg, 0, T) + head_flops_per_row
+        result["prefill"] = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
+                             "frac": round(flops / psec / PEAK_FLOPS[short], 4)}
+        log(f"prefill {T} tokens: {psec * 1e3:.2f} ms, {T / psec:.0f} tok/s")
+    if not args.no_points:
+        points = {}
+        for b in (1, 64):
+            s = decode_point(b, max(8, args.steps // 2), max(2, args.warmup // 2))
+            points[f"decode_b{b}"] = round(b / s, 2)
+        result["points"] = points
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

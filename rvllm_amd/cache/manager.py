@@ -150,6 +150,24 @@ class CacheManager:
             if n:
                 rc.tables[name].extend(self.groups[name].pool.take(request, n))
 
+    def adopt_length(self, request: Hashable, length: int) -> None:
+        """Make a fresh request hold ``length`` tokens without running them:
+        it gets exactly the pages a request of that length holds (none behind
+        a window).  For measurements on a cache filled by hand."""
+        rc = self.requests[request]
+        if rc.length != 0 or any(rc.tables[name] for name in self.groups):
+            raise ValueError("only a fresh request can adopt a length")
+        plan = {}
+        for name, g in self.groups.items():
+            first = g.first_kept_page(length)
+            count = -(-length // g.page_size) - first
+            if count > g.pool.free_count:
+                raise OutOfPages(name, count, g.pool.free_count)
+            plan[name] = (first, count)
+        for name, (first, count) in plan.items():
+            rc.tables[name] = [-1] * first + self.groups[name].pool.take(request, count)
+        rc.length = length
+
     def commit(self, request: Hashable, new_length: int) -> None:
         """The step that wrote the positions up to ``new_length`` is done:
         record the length and give back the pages the window has passed."""
