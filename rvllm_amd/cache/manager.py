@@ -4,10 +4,8 @@ Layers are grouped by what they need to keep.  Layers whose tokens see every
 earlier key form one group, layers with a window of W form another; each
 group has a pool of pages of its own and, for every live request, one block
 table (logical page -> physical page) that all layers of the group share.
-Every layer of a group has key and value storage of its own,
-``[num_pages, page_size, kv_heads, head_dim]`` (the reference's layout:
-v3/crates/rvllm-mem/src/kv_layout.rs:1-46), addressed through the group's
-table.  A window group gives a page back as soon as every position on it has
+Every layer of a group has key and value storage of its own (its layout is the
+storage's matter), addressed through the group's table.  A window group gives a page back as soon as every position on it has
 left the window of the request's next token.  Mixers with a state of fixed size get a
 slot per request instead of pages.
 

@@ -1,9 +1,12 @@
 """Device memory behind the cache manager's books.
 
-Every layer with a key/value need gets one tensor
-``[2, num_pages, page_size, kv_heads, head_dim]``, keys then values
-(v3/crates/rvllm-mem/src/kv_layout.rs:1-46); every layer with a fixed-size
-state gets ``[max_requests, *shape]``.  Nothing is cleared when pages change
+Every layer with a key/value need gets one allocation, keys then values (as
+in v3/crates/rvllm-mem/src/kv_layout.rs:1-46).  Inside it keys are
+``[num_pages, kv_heads, page_size, head_dim]`` and values are transposed
+inside the page, ``[num_pages, kv_heads, head_dim, page_size]``: what one
+key/value head holds on a page is one contiguous block, and the matrix-core
+attention kernel reads both operands in the order it sums them.  Every layer
+with a fixed-size state gets ``[max_requests, *shape]``.  Nothing is cleared when pages change
 hands: a position that a token may not see is never read, so what an earlier
 request left behind is unreachable (the reference relies on the same for its
 rejected drafts: v3/crates/rvllm-runtime/src/gemma4_bring_up.rs:4237-4243).
@@ -30,10 +33,12 @@ class CacheStorage:
         for i, need in enumerate(manager.needs):
             if isinstance(need, KVNeed):
                 g = manager.groups[manager.layer_group[i]]
-                kv = torch.zeros((2, g.pool.num_pages, g.page_size, need.num_kv_heads, need.head_dim), dtype=dtype,
+                kv = torch.zeros((2, g.pool.num_pages, need.num_kv_heads, g.page_size * need.head_dim), dtype=dtype,
                                  device=self.device)
                 self.bytes += kv.numel() * kv.element_size()
-                self.views.append(KVCacheView(kv[0], kv[1], g.name, g.page_size))
+                keys = kv[0].view(g.pool.num_pages, need.num_kv_heads, g.page_size, need.head_dim)
+                values = kv[1].view(g.pool.num_pages, need.num_kv_heads, need.head_dim, g.page_size)
+                self.views.append(KVCacheView(keys, values, g.name, g.page_size))
             elif isinstance(need, StateNeed):
                 slots = torch.zeros((manager.max_requests, *need.shape), dtype=need.dtype, device=self.device)
                 self.bytes += slots.numel() * slots.element_size()

@@ -20,6 +20,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "kv_layout.h"
 
 #define ATT_MAX_HD 512
 #define ATT_DIMS_PER_LANE (ATT_MAX_HD / RV_WAVE)
@@ -32,7 +33,7 @@ __global__ void paged_attention_generic_kernel(const T* __restrict__ q, const T*
                                                int hd, int page_size, int num_pages, int window, float scale) {
   __shared__ float q_s[ATT_MAX_HD];
   __shared__ float p_s[RV_WAVE];
-  __shared__ int row_s[RV_WAVE];
+  __shared__ int page_s[RV_WAVE];
 
   const int lane = threadIdx.x;
   const int t = blockIdx.x / nq;
@@ -55,13 +56,13 @@ __global__ void paged_attention_generic_kernel(const T* __restrict__ q, const T*
   for (int start = lo; start <= p; start += RV_WAVE) {
     const int j = start + lane;
     float s = -INFINITY;
-    int row = -1;
+    int my_page = -1;
     if (j <= p) {
       const int logical = j / page_size;
       const int page = logical < table_width ? table[logical] : -1;
       if (page >= 0 && page < num_pages) {
-        row = page * page_size + (j % page_size);
-        const T* kr = k_pages + ((size_t)row * nkv + kvh) * hd;
+        my_page = page;
+        const T* kr = k_pages + rv_k_index(page, kvh, j % page_size, 0, nkv, page_size, hd);
         float dot = 0.f;
         for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], rv_to_float(kr[d]), dot);
         s = dot * scale;
@@ -75,9 +76,9 @@ __global__ void paged_attention_generic_kernel(const T* __restrict__ q, const T*
     const float corr = expf(m - m_new);  // 0 on the first tile (m = -inf)
     l = l * corr + rv_wave_sum(pj);
     m = m_new;
-    __syncthreads();  // the previous tile's p_s / row_s are no longer read
+    __syncthreads();  // the previous tile's p_s / page_s are no longer read
     p_s[lane] = pj;
-    row_s[lane] = row;
+    page_s[lane] = my_page;
     __syncthreads();
     const int count = (p - start + 1 < RV_WAVE) ? p - start + 1 : RV_WAVE;
 #pragma unroll
@@ -86,8 +87,9 @@ __global__ void paged_attention_generic_kernel(const T* __restrict__ q, const T*
       if (d < hd) {
         float a = acc[i] * corr;
         for (int jj = 0; jj < count; ++jj) {
-          const int r = row_s[jj];
-          const float v = r >= 0 ? rv_to_float(v_pages[((size_t)r * nkv + kvh) * hd + d]) : 0.f;
+          const int pg = page_s[jj];
+          const float v =
+              pg >= 0 ? rv_to_float(v_pages[rv_v_index(pg, kvh, (start + jj) % page_size, d, nkv, page_size, hd)]) : 0.f;
           a = fmaf(p_s[jj], v, a);
         }
         acc[i] = a;

@@ -1,0 +1,4 @@
+// Matrix-core attention for head sizes 80, 96, 112 and 128 (see attention_mfma.inc).
+#define RV_ATTN_ENTRY rv_attn_mfma_g1
+#define RV_ATTN_CASES RV_ATTN_CASE(80) RV_ATTN_CASE(96) RV_ATTN_CASE(112) RV_ATTN_CASE(128)
+#include "attention_mfma.inc"

@@ -10,11 +10,13 @@
 //               x'[i+hd/2] = x[i]*sin + x[i+hd/2]*cos
 //             angle = float(pos) * inv_freq[i]  (v3/kernels/fused_rope_partial_f16kv.cu:50-65,
 //             metal_host.rs:1160-1166); dimensions past rot/2 pass through
-//   write     K (normed, rotated) and V (as projected) go to
-//             pages[page, pos % page_size, kv_head, :], page = table[req, pos / page_size]
-//             (layout: fused_rope_partial_f16kv.cu:69-91); a negative page skips the write
+//   write     K (normed, rotated) and V (as projected) go to slot pos % page_size of
+//             page = table[req, pos / page_size], in the layout of kv_layout.h
+//             (the reference writes at the same point: fused_rope_partial_f16kv.cu:69-91);
+//             a negative page skips the write
 // Norm, angle, sine and cosine are 32-bit.
 #include "common.h"
+#include "kv_layout.h"
 
 #define QKR_MAX_HD 512
 
@@ -49,14 +51,15 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
     if (logical >= table_width) return;
     const int page = block_table[(size_t)req * table_width + logical];
     if (page < 0 || page >= num_pages) return;
-    const int kvh = is_k ? head - nq : head - nq - nkv;
-    T* base = is_k ? k_pages : v_pages;
-    dst = base + (((size_t)page * page_size + (pos % page_size)) * nkv + kvh) * hd;
-  }
-
-  if (!is_q && !is_k) {  // values are stored as projected
-    for (int d = lane; d < hd; d += RV_WAVE) dst[d] = src[d];
-    return;
+    const int slot = pos % page_size;
+    if (is_k) {
+      dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
+    } else {
+      // values are stored as projected, transposed inside the page
+      T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
+      for (int d = lane; d < hd; d += RV_WAVE) col[(size_t)d * page_size] = src[d];
+      return;
+    }
   }
 
   float* x = buf[wave];

@@ -43,7 +43,7 @@ def _sources() -> list[Path]:
 
 
 def _headers() -> list[Path]:
-    return sorted(CSRC.glob("*.h"))
+    return sorted(list(CSRC.glob("*.h")) + list(CSRC.glob("*.inc")))
 
 
 def source_hash() -> str:

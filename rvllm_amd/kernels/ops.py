@@ -88,6 +88,18 @@ def _i32(*tensors: torch.Tensor) -> None:
 _c_int, _c_float, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_longlong
 
 
+def _cache_geometry(k_pages: torch.Tensor, v_pages: torch.Tensor, what: str) -> tuple[int, int, int, int]:
+    """(pages, kv heads, page size, head size) of a layer's cache: keys are
+    ``[pages, kv_heads, page_size, head_dim]``, values are transposed inside
+    the page, ``[pages, kv_heads, head_dim, page_size]``."""
+    _need(k_pages.dim() == 4 and v_pages.dim() == 4, f"{what}: cache pages must have four dimensions")
+    num_pages, nkv, page_size, hd = k_pages.shape
+    _need(tuple(v_pages.shape) == (num_pages, nkv, hd, page_size),
+          f"{what}: keys are {tuple(k_pages.shape)}, so values must be {(num_pages, nkv, hd, page_size)}, "
+          f"got {tuple(v_pages.shape)}")
+    return num_pages, nkv, page_size, hd
+
+
 # --------------------------------------------------------------------------
 def embed_gather(table: torch.Tensor, ids: torch.Tensor, scale: float, out: torch.Tensor) -> torch.Tensor:
     _gpu(table, ids, out)
@@ -211,8 +223,8 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
     if write_kv:
         _need(k_pages is not None and v_pages is not None and block_table is not None, "qk_norm_rope: no cache given")
         _i32(block_table)
-        num_pages, page_size, nkv, hd = k_pages.shape
-        _need((nkv, hd) == (num_kv_heads, head_dim) and v_pages.shape == k_pages.shape, "qk_norm_rope: bad page shape")
+        num_pages, nkv, page_size, hd = _cache_geometry(k_pages, v_pages, "qk_norm_rope")
+        _need((nkv, hd) == (num_kv_heads, head_dim), "qk_norm_rope: cache pages do not fit the heads")
         _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "qk_norm_rope: cache dtype differs")
         width = block_table.shape[1]
     _check(library().rv_qk_norm_rope_kv_write(
@@ -230,11 +242,10 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     _gpu(q, k_pages, v_pages, block_table, positions, token_req, out)
     _i32(block_table, positions, token_req)
     n = q.shape[0]
-    num_pages, page_size, nkv, hd = k_pages.shape
+    num_pages, nkv, page_size, hd = _cache_geometry(k_pages, v_pages, "attention")
     _need(q.shape == (n, num_q_heads * hd), f"attention: q is {tuple(q.shape)}, expected {(n, num_q_heads * hd)}")
     _need(out.shape == q.shape and out.dtype == q.dtype, "attention: out must match q")
-    _need(v_pages.shape == k_pages.shape and k_pages.dtype == q.dtype and v_pages.dtype == q.dtype,
-          "attention: cache must match q")
+    _need(k_pages.dtype == q.dtype and v_pages.dtype == q.dtype, "attention: cache must match q")
     _need(positions.numel() >= n and token_req.numel() >= n, "attention: positions/token_req too short")
     _check(library().rv_paged_attention_generic(
         _stream(), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _c_int(block_table.shape[1]),
@@ -248,9 +259,83 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
     """Attention of the step's tokens over the cache; picks the kernel.
 
     The 32-bit path always runs the generic kernel.  bf16 runs the
-    matrix-core kernels where one covers the head size, else the generic one."""
+    matrix-core kernel where it covers the head size and grouping, else the
+    generic one."""
+    if q.dtype == torch.bfloat16 and mfma_attention_covers(k_pages, v_pages, num_q_heads):
+        return paged_attention_mfma(q, k_pages, v_pages, block_table, step, out, num_q_heads, scale, window)
     return paged_attention_generic(q, k_pages, v_pages, block_table, step.positions, step.token_req, out,
                                    num_q_heads, scale, window)
+
+
+MFMA_ATTENTION_MAX_HEAD_DIM = 256
+MFMA_ATTENTION_MAX_GROUP = 16
+# Waves that fill the chip: 256 CUs, 4 SIMDs each, two waves a SIMD.
+_ATTENTION_TARGET_UNITS = 2048
+
+
+def mfma_attention_covers(k_pages: torch.Tensor, v_pages: torch.Tensor, num_q_heads: int) -> bool:
+    _, nkv, page_size, hd = k_pages.shape
+    return (hd % 16 == 0 and hd <= MFMA_ATTENTION_MAX_HEAD_DIM and page_size % 16 == 0
+            and num_q_heads % nkv == 0 and num_q_heads // nkv <= MFMA_ATTENTION_MAX_GROUP)
+
+
+def plan_attention_splits(num_requests: int, max_portion: int, max_context: int, nkv: int, group: int,
+                          window: Optional[int]) -> tuple[int, int, int]:
+    """(tiles per request, number of key splits, keys per split) for the
+    matrix-core kernel.  A tile is 16 / group_pad tokens of one request and one
+    key/value head; its keys are split so that about 2048 waves run."""
+    group_pad = 1
+    while group_pad < group:
+        group_pad *= 2
+    tokens_per_tile = 16 // group_pad
+    tiles = -(-max_portion // tokens_per_tile)
+    span = max_context
+    if window:
+        # first key of a tile rounded down to 32, up to the tile's last token
+        span = min(span, window - 1 + 31 + tokens_per_tile)
+    span = -(-span // 32) * 32
+    units = num_requests * tiles * nkv
+    splits = 1 if units >= 512 else min(-(-_ATTENTION_TARGET_UNITS // units), span // 32)
+    split_len = -(-(-(-span // splits)) // 32) * 32
+    return tiles, -(-span // split_len), split_len
+
+
+def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                         step, out: torch.Tensor, num_q_heads: int, scale: float, window: Optional[int],
+                         splits: Optional[tuple[int, int]] = None) -> torch.Tensor:
+    """bf16 attention on the matrix cores.  ``splits`` = (number, keys per
+    split) overrides the plan (tests use it to force every path)."""
+    _gpu(q, k_pages, v_pages, block_table, out)
+    _i32(block_table)
+    n = q.shape[0]
+    num_pages, nkv, page_size, hd = _cache_geometry(k_pages, v_pages, "attention")
+    _need(q.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16,
+          "attention (matrix cores): bfloat16 only")
+    _need(mfma_attention_covers(k_pages, v_pages, num_q_heads),
+          f"attention (matrix cores): head_dim {hd} must be a multiple of 16 up to {MFMA_ATTENTION_MAX_HEAD_DIM}, "
+          f"at most {MFMA_ATTENTION_MAX_GROUP} query heads per key/value head, pages a multiple of 16")
+    _need(q.shape == (n, num_q_heads * hd) and out.shape == q.shape and out.dtype == q.dtype,
+          "attention (matrix cores): bad q or out shape")
+    _need(n == step.num_tokens, "attention (matrix cores): q must hold the step's tokens")
+    group = num_q_heads // nkv
+    tiles, num_splits, split_len = plan_attention_splits(step.num_requests, step.max_portion, step.max_context, nkv,
+                                                         group, window)
+    if splits is not None:
+        num_splits, split_len = splits
+        need = -(-step.max_context // 32) * 32
+        _need(window is not None or num_splits * split_len >= need, "attention: the splits do not cover the context")
+    part_o = part_ml = None
+    if num_splits > 1:
+        units = step.num_requests * tiles * nkv * num_splits
+        part_o = torch.empty(units * 16 * hd, dtype=torch.float32, device=q.device)
+        part_ml = torch.empty(units * 32, dtype=torch.float32, device=q.device)
+    entry = getattr(library(), f"rv_attn_mfma_g{(hd // 16 - 1) // 4}")
+    _check(entry(_stream(), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _c_int(block_table.shape[1]),
+                 _ptr(step.q_start), _ptr(step.chunk_start), _ptr(step.token_req), _ptr(out), _ptr(part_o),
+                 _ptr(part_ml), _c_int(n), _c_int(step.num_requests), _c_int(tiles), _c_int(num_q_heads), _c_int(nkv),
+                 _c_int(hd), _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_int(num_splits),
+                 _c_int(split_len), _c_float(scale)))
+    return out
 
 
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:

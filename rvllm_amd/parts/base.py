@@ -75,10 +75,11 @@ CacheNeed = "KVNeed | StateNeed | None"
 
 @dataclasses.dataclass
 class KVCacheView:
-    """What an attention-like mixer gets for its layer: the key and value
-    pages ``[num_pages, page_size, num_kv_heads, head_dim]`` and the name of
-    the group whose block table addresses them.  ``writes`` is False for a
-    layer that reads another layer's cache."""
+    """What an attention-like mixer gets for its layer: the key pages
+    ``[num_pages, num_kv_heads, page_size, head_dim]``, the value pages
+    ``[num_pages, num_kv_heads, head_dim, page_size]`` (transposed inside the
+    page) and the name of the group whose block table addresses them.
+    ``writes`` is False for a layer that reads another layer's cache."""
 
     k_pages: torch.Tensor
     v_pages: torch.Tensor

@@ -4,6 +4,7 @@ vocabularies that are no power of two, head sizes in steps of 16, odd head
 groupings, pages of every size."""
 
 import math
+import types
 
 import pytest
 import torch
@@ -141,6 +142,17 @@ def paged_setup(T_total, nkv, hd, page_size, dtype, seed, scramble=True):
     return g, k_pages, v_pages, table
 
 
+def to_cache(k_pages, v_pages):
+    """The test keeps pages as [page, slot, kv_head, d]; the cache on the
+    device holds keys as [page, kv_head, slot, d] and values transposed inside
+    the page, [page, kv_head, d, slot]."""
+    return dev(k_pages.permute(0, 2, 1, 3)), dev(v_pages.permute(0, 2, 3, 1))
+
+
+def from_cache(kp, vp):
+    return kp.cpu().permute(0, 2, 1, 3), vp.cpu().permute(0, 3, 1, 2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,hd,rot", [(4, 2, 16, 16), (6, 3, 48, 48), (5, 1, 80, 40), (8, 4, 256, 256), (3, 3, 128, 0)])
 @pytest.mark.parametrize("page_size", [16, 64])
@@ -153,9 +165,11 @@ def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size):
     positions = torch.arange(90, 90 + T, dtype=torch.int32)  # straddles page edges
     inv_freq = (10000.0 ** (-2.0 * torch.arange(rot // 2, dtype=torch.float64) / hd) / 4.0).float()
     q_out = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
-    kp, vp = dev(k_pages), dev(v_pages)
+    kp_dev, vp_dev = to_cache(k_pages, v_pages)
     ops.qk_norm_rope_kv_write(dev(qkv), q_out, dev(qw), dev(kw), 1e-6, 1.0, dev(inv_freq) if rot else None, rot,
-                              dev(positions), dev(torch.zeros(T, dtype=torch.int32)), dev(table), kp, vp, nq, nkv, hd)
+                              dev(positions), dev(torch.zeros(T, dtype=torch.int32)), dev(table), kp_dev, vp_dev, nq,
+                              nkv, hd)
+    kp, vp = from_cache(kp_dev, vp_dev)
     q, k, v = qkv.double().split([nq * hd, nkv * hd, nkv * hd], dim=1)
     q = P.rmsnorm(q.view(T, nq, hd), qw.double(), 1e-6)
     k = P.rmsnorm(k.view(T, nkv, hd), kw.double(), 1e-6)
@@ -182,7 +196,7 @@ def test_qk_norm_rope_without_cache_write_leaves_the_cache_alone():
     g, k_pages, v_pages, table = paged_setup(64, nkv, hd, 16, torch.float32, 8)
     qkv = torch.randn(T, (nq + 2 * nkv) * hd, generator=g)
     q_out = torch.empty(T, nq * hd, device=DEV)
-    kp, vp = dev(k_pages), dev(v_pages)
+    kp, vp = to_cache(k_pages, v_pages)
     ops.qk_norm_rope_kv_write(dev(qkv), q_out, None, None, 0.0, 0.0, None, 0, dev(torch.arange(T, dtype=torch.int32)),
                               dev(torch.zeros(T, dtype=torch.int32)), dev(table), kp, vp, nq, nkv, hd, write_kv=False)
     assert kp.abs().sum() == 0 and vp.abs().sum() == 0
@@ -203,69 +217,158 @@ def reference_attention(q, k_all, v_all, positions, scale, window):
     return out
 
 
+class Case:
+    """Requests with their portions, a scrambled paged cache and the flat batch."""
+
+    def __init__(self, portions, nq, nkv, hd, page_size, dtype, seed, window=None, drop_passed_pages=True):
+        # portions: (position of the first query token, number of query tokens) per request
+        g = torch.Generator().manual_seed(seed)
+        self.nq, self.nkv, self.hd, self.page_size, self.window, self.dtype = nq, nkv, hd, page_size, window, dtype
+        self.portions = portions
+        B = len(portions)
+        lengths = [s + n for s, n in portions]
+        pages_per = [-(-L // page_size) for L in lengths]
+        n_pages = sum(pages_per) + 5
+        order = torch.randperm(n_pages, generator=g).tolist()
+        self.k_log = torch.zeros(n_pages, page_size, nkv, hd, dtype=dtype)  # [page, slot, head, d]
+        self.v_log = torch.zeros_like(self.k_log)
+        self.table = torch.full((B, max(pages_per) + 2), -1, dtype=torch.int32)
+        self.k_all, self.v_all = [], []
+        nxt = 0
+        for b, L in enumerate(lengths):
+            k = torch.randn(L, nkv, hd, generator=g).to(dtype)
+            v = torch.randn(L, nkv, hd, generator=g).to(dtype)
+            self.k_all.append(k)
+            self.v_all.append(v)
+            for i in range(pages_per[b]):
+                page = order[nxt]
+                nxt += 1
+                self.table[b, i] = page
+                rows = slice(i * page_size, min((i + 1) * page_size, L))
+                self.k_log[page, : rows.stop - rows.start] = k[rows]
+                self.v_log[page, : rows.stop - rows.start] = v[rows]
+            if window and drop_passed_pages:
+                # pages that the window of the portion's first token has passed are gone:
+                # a kernel that touches them reads NaN
+                first = max(0, portions[b][0] - window + 1) // page_size
+                for i in range(first):
+                    self.k_log[int(self.table[b, i])] = float("nan")
+                    self.v_log[int(self.table[b, i])] = float("nan")
+                    self.table[b, i] = -1
+        T = sum(n for _, n in portions)
+        self.q = torch.randn(T, nq, hd, generator=g).to(dtype)
+        self.positions = torch.cat([torch.arange(s, s + n, dtype=torch.int32) for s, n in portions])
+        self.token_req = torch.cat([torch.full((n,), b, dtype=torch.int32) for b, (_, n) in enumerate(portions)])
+        starts = [0]
+        for _, n in portions:
+            starts.append(starts[-1] + n)
+        self.step = types.SimpleNamespace(
+            num_tokens=T, num_requests=B, positions=dev(self.positions), token_req=dev(self.token_req),
+            q_start=dev(torch.tensor(starts, dtype=torch.int32)),
+            chunk_start=dev(torch.tensor([s for s, _ in portions], dtype=torch.int32)),
+            max_portion=max(n for _, n in portions), max_context=max(lengths))
+
+    def reference(self, scale):
+        outs = []
+        t = 0
+        for b, (s, n) in enumerate(self.portions):
+            pos = torch.arange(s, s + n)
+            outs.append(reference_attention(self.q[t:t + n].double(), self.k_all[b].double(), self.v_all[b].double(),
+                                            pos, scale, self.window))
+            t += n
+        return torch.cat(outs)
+
+    def run(self, kernel, scale, **kw):
+        kp, vp = to_cache(self.k_log, self.v_log)
+        T = self.q.shape[0]
+        out = torch.full((T, self.nq * self.hd), float("nan"), dtype=self.dtype, device=DEV)
+        q = dev(self.q.view(T, -1))
+        if kernel == "generic":
+            ops.paged_attention_generic(q, kp, vp, dev(self.table), self.step.positions, self.step.token_req, out,
+                                        self.nq, scale, self.window)
+        else:
+            ops.paged_attention_mfma(q, kp, vp, dev(self.table), self.step, out, self.nq, scale, self.window, **kw)
+        return out.cpu().view(T, self.nq, self.hd)
+
+
+MIXED = [(150, 53), (180, 1), (0, 40), (202, 1), (31, 2)]  # portions beside single tokens, page edges, position 0
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,hd", [(4, 2, 16), (6, 1, 48), (3, 3, 80), (8, 4, 256), (2, 1, 128)])
 @pytest.mark.parametrize("window", [None, 7, 100])
 def test_paged_attention_generic(dtype, nq, nkv, hd, window):
-    ctx, page_size = 203, 16
-    g, k_pages, v_pages, table = paged_setup(ctx, nkv, hd, page_size, dtype, 9)
-    k_all = torch.randn(ctx, nkv, hd, generator=g).to(dtype)
-    v_all = torch.randn(ctx, nkv, hd, generator=g).to(dtype)
-    for j in range(ctx):
-        page, off = int(table[0, j // page_size]), j % page_size
-        k_pages[page, off], v_pages[page, off] = k_all[j], v_all[j]
-    # pages behind the window are gone: a kernel that touches them fails loudly
-    if window:
-        first_needed = max(0, 150 - window + 1) // page_size
-        for i in range(first_needed):
-            k_pages[int(table[0, i])] = float("nan")
-            table[0, i] = -1
-    positions = torch.tensor([150, 151, 160, 175, 176, 191, 192, 202], dtype=torch.int32)
-    q = torch.randn(len(positions), nq, hd, generator=g).to(dtype)
-    out = torch.empty(len(positions), nq * hd, dtype=dtype, device=DEV)
-    ops.paged_attention_generic(dev(q.view(len(positions), -1)), dev(k_pages), dev(v_pages), dev(table),
-                                dev(positions), dev(torch.zeros(len(positions), dtype=torch.int32)), out, nq,
-                                hd ** -0.5, window)
-    want = reference_attention(q.double(), k_all.double(), v_all.double(), positions, hd ** -0.5, window)
-    assert torch.allclose(out.cpu().float().view_as(want), want.float(), **tol(dtype))
+    case = Case(MIXED, nq, nkv, hd, 16, dtype, 9, window)
+    got = case.run("generic", hd ** -0.5)
+    assert torch.allclose(got.float(), case.reference(hd ** -0.5).float(), **tol(dtype))
 
 
-def test_paged_attention_finds_one_far_key_among_hundreds():
+@pytest.mark.parametrize("nq,nkv,hd", [(4, 2, 16), (6, 1, 48), (3, 3, 80), (8, 4, 256), (2, 1, 128), (16, 1, 32),
+                                       (5, 5, 240), (12, 4, 64)])
+@pytest.mark.parametrize("window", [None, 7, 100])
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_paged_attention_mfma(nq, nkv, hd, window, page_size):
+    case = Case(MIXED, nq, nkv, hd, page_size, torch.bfloat16, 9, window)
+    want = case.reference(hd ** -0.5).float()
+    assert torch.allclose(case.run("mfma", hd ** -0.5).float(), want, **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("splits", [(1, 224), (2, 128), (7, 32), (4, 64)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_paged_attention_mfma_every_split(splits, window):
+    """One split, splits that end on and off page edges, splits that are empty
+    for some tiles: all give the same result."""
+    case = Case(MIXED, 8, 4, 256, 16, torch.bfloat16, 10, window)
+    want = case.reference(1.0 / 16).float()
+    assert torch.allclose(case.run("mfma", 1.0 / 16, splits=splits).float(), want, **tol(torch.bfloat16))
+
+
+def test_paged_attention_mfma_long_decode_batch():
+    """Decode shapes: many requests with one token each at long, different contexts."""
+    portions = [(4000 + 37 * i, 1) for i in range(9)]
+    for window in (None, 1024):
+        case = Case(portions, 8, 4, 256, 16, torch.bfloat16, 11, window)
+        want = case.reference(1.0 / 16).float()
+        assert torch.allclose(case.run("mfma", 1.0 / 16).float(), want, **tol(torch.bfloat16))
+
+
+def test_mfma_attention_says_what_it_does_not_cover():
+    case = Case([(5, 1)], 34, 2, 32, 16, torch.bfloat16, 12)  # 17 query heads per key/value head
+    with pytest.raises(ops.KernelError, match="at most 16 query heads"):
+        case.run("mfma", 1.0)
+    assert not ops.mfma_attention_covers(*to_cache(case.k_log, case.v_log), 34)
+
+
+@pytest.mark.parametrize("kernel,dtype", [("generic", torch.float32), ("generic", torch.bfloat16),
+                                          ("mfma", torch.bfloat16)])
+def test_paged_attention_finds_one_far_key_among_hundreds(kernel, dtype):
     """Random keys hide a wrong mask or table; here one far key carries all
     the weight, so the output is its value exactly."""
-    nq, nkv, hd, ctx, page_size = 2, 1, 32, 700, 16
-    g, k_pages, v_pages, table = paged_setup(ctx, nkv, hd, page_size, torch.float32, 10)
-    k_all = torch.randn(ctx, nkv, hd, generator=g) * 0.01
-    v_all = torch.randn(ctx, nkv, hd, generator=g)
+    nq, nkv, hd, ctx = 2, 1, 32, 700
     far = 17  # on the second page
-    k_all[far, 0] = 0
-    k_all[far, 0, 3] = 40.0
-    for j in range(ctx):
-        k_pages[int(table[0, j // page_size]), j % page_size] = k_all[j]
-        v_pages[int(table[0, j // page_size]), j % page_size] = v_all[j]
-    q = torch.zeros(1, nq, hd)
-    q[0, :, 3] = 40.0
-    out = torch.empty(1, nq * hd, device=DEV)
-    args = (dev(q.view(1, -1)), dev(k_pages), dev(v_pages), dev(table), dev(torch.tensor([ctx - 1], dtype=torch.int32)),
-            dev(torch.zeros(1, dtype=torch.int32)), out, nq, 1.0)
-    ops.paged_attention_generic(*args, None)
-    assert torch.allclose(out.cpu().view(nq, hd), v_all[far, 0].expand(nq, hd), atol=1e-5)
-    # exactly at the window's edge the key is still seen, one further it is not
-    ops.paged_attention_generic(*args, ctx - far)
-    assert torch.allclose(out.cpu().view(nq, hd), v_all[far, 0].expand(nq, hd), atol=1e-5)
-    ops.paged_attention_generic(*args, ctx - far - 1)
-    assert not torch.allclose(out.cpu().view(nq, hd), v_all[far, 0].expand(nq, hd), atol=1e-2)
+    for window, found in ((None, True), (ctx - far, True), (ctx - far - 1, False)):
+        # exactly at the window's edge the key is still seen, one further it is not
+        case = Case([(ctx - 1, 1)], nq, nkv, hd, 16, dtype, 10, window, drop_passed_pages=False)
+        k, v = case.k_all[0], case.v_all[0]
+        k *= 0.01
+        k[far, 0] = 0
+        k[far, 0, 3] = 40.0
+        page, slot = int(case.table[0, far // 16]), far % 16
+        case.k_log[:] = 0
+        for j in range(ctx):
+            case.k_log[int(case.table[0, j // 16]), j % 16] = k[j]
+        case.q[:] = 0
+        case.q[0, :, 3] = 40.0
+        got = case.run(kernel, 1.0).float()
+        same = torch.allclose(got[0], v[far, 0].float().expand(nq, hd), atol=2e-2 if dtype == torch.bfloat16 else 1e-5)
+        assert same == found, (window, found)
 
 
-def test_paged_attention_missing_page_shows():
-    nq, nkv, hd = 1, 1, 16
-    g, k_pages, v_pages, table = paged_setup(40, nkv, hd, 16, torch.float32, 11)
-    table[0, 1] = -1  # a visible page is missing: the result must not look valid
-    q = torch.randn(1, hd, generator=g)
-    out = torch.empty(1, hd, device=DEV)
-    ops.paged_attention_generic(dev(q), dev(k_pages), dev(v_pages), dev(table), dev(torch.tensor([39], dtype=torch.int32)),
-                                dev(torch.zeros(1, dtype=torch.int32)), out, nq, 1.0, None)
-    assert torch.isnan(out).all()
+@pytest.mark.parametrize("kernel,dtype", [("generic", torch.float32), ("mfma", torch.bfloat16)])
+def test_paged_attention_missing_page_shows(kernel, dtype):
+    case = Case([(39, 1)], 1, 1, 16, 16, dtype, 11)
+    case.table[0, 1] = -1  # a visible page is missing: the result must not look valid
+    assert torch.isnan(case.run(kernel, 1.0)).all()
 
 
 @pytest.mark.parametrize("vocab", [5, 256, 509, 4097, 262208])
