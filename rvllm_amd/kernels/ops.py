@@ -367,5 +367,32 @@ def topk_select(logits: torch.Tensor, k: int, inv_temp: torch.Tensor) -> tuple[t
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optional[torch.Tensor]:
     """out = x @ w^T on the matrix cores for bf16 inputs; None when no
-    hand-written kernel covers the shape (the caller then uses another path)."""
-    return None
+    hand-written kernel covers the shape (the caller then uses another path).
+
+    Products with up to 64 rows run the kernel that is built around reading
+    ``w`` once.  A 32-bit result of more rows (logits at many positions) runs
+    it over blocks of 64 rows; a bf16 result of more rows is left to the
+    library product."""
+    m, k = x.shape
+    n = w.shape[0]
+    if k % 8 or x.stride(1) != 1 or w.stride(1) != 1 or out.stride(1) != 1:
+        return None
+    if (m > 1 and x.stride(0) % 8) or (n > 1 and w.stride(0) % 8) or x.data_ptr() % 16 or w.data_ptr() % 16:
+        return None
+    if m > SKINNY_MAX_ROWS and out.dtype != torch.float32:
+        return None
+    _need(x.is_cuda and w.is_cuda and out.is_cuda, "gemm: arguments must live on the GPU")
+    _need(out.shape == (m, n) and w.shape[1] == k, "gemm: shapes do not fit")
+    lib = library()
+    ldx = x.stride(0) if m > 1 else k
+    ldw = w.stride(0) if n > 1 else k
+    ldc = out.stride(0) if m > 1 else n
+    for m0 in range(0, m, SKINNY_MAX_ROWS):
+        rows = min(SKINNY_MAX_ROWS, m - m0)
+        _check(lib.rv_gemm_skinny(_stream(), ctypes.c_void_p(x.data_ptr() + m0 * ldx * 2), _ptr(w),
+                                  ctypes.c_void_p(out.data_ptr() + m0 * ldc * out.element_size()), _dt(out),
+                                  _c_int(rows), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(ldc)))
+    return out
+
+
+SKINNY_MAX_ROWS = 64

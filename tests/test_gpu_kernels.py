@@ -129,6 +129,41 @@ def test_gemm_plain_bf16_inputs_give_32_bit_logits():
     assert torch.allclose(out.cpu(), a.float() @ w.float().T, atol=1e-4, rtol=1e-5)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 4096, 2560), (17, 509, 96), (64, 2560, 10240), (33, 100, 2048),
+                                   (3, 20480, 2560), (16, 7, 8), (200, 301, 80)])
+def test_gemm_skinny(m, n, k, out_dtype):
+    g = torch.Generator().manual_seed(20)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    out = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+    got = ops.gemm_bf16(dev(x), dev(w), out)
+    if m > 64 and out_dtype == torch.bfloat16:
+        assert got is None  # left to the library product
+        return
+    assert got is out
+    want = x.double() @ w.double().T
+    err = (out.cpu().double() - want).abs().max().item()
+    scale = want.abs().max().item()
+    assert err <= (2e-6 if out_dtype == torch.float32 else 5e-3) * scale * max(1.0, math.sqrt(k) / 16)
+    # a row gives the same bits alone as in the batch
+    one = torch.empty((1, n), dtype=out_dtype, device=DEV)
+    ops.gemm_bf16(dev(x[m - 1:m]), dev(w), one)
+    assert torch.equal(one[0], out[m - 1])
+
+
+def test_gemm_skinny_reads_strided_rows_and_refuses_what_it_cannot():
+    g = torch.Generator().manual_seed(21)
+    big = dev(torch.randn(6, 96, generator=g).bfloat16())
+    x = big[:, :64]  # rows 96 apart
+    w = dev(torch.randn(40, 64, generator=g).bfloat16())
+    out = torch.empty((6, 40), dtype=torch.float32, device=DEV)
+    assert ops.gemm_bf16(x, w, out) is out
+    assert torch.allclose(out.cpu(), x.cpu().float() @ w.cpu().float().T, atol=1e-3)
+    assert ops.gemm_bf16(dev(torch.zeros(2, 12).bfloat16()), dev(torch.zeros(4, 12).bfloat16()),
+                         torch.empty((2, 4), dtype=torch.float32, device=DEV)) is None  # K is no multiple of 8
+
+
 def paged_setup(T_total, nkv, hd, page_size, dtype, seed, scramble=True):
     """A cache whose pages are handed out in a scrambled order."""
     g = torch.Generator().manual_seed(seed)
