@@ -3,21 +3,25 @@
 // 32-bit output.  The time of such a product is the time to read W once, so the
 // kernel is laid out around that read:
 //
-//   * a wave owns 16 rows of W and a slice of K; the waves of a block are the
-//     K-slices of the same 16 rows, so that even a matrix with few rows keeps
-//     every CU busy;
-//   * W is the A operand of MFMA 16x16x32 (16 rows x 32 k): a lane reads 64
-//     contiguous bytes of its row per step (four 16-byte loads, four MFMAs), the
-//     four lanes of a row together 256 contiguous bytes; nothing passes
-//     through LDS;
-//   * x is the B operand, read from L2 (it is a few tens of kilobytes); up to
-//     four column sets of 16 rows of x share each read of W;
-//   * the partial sums of the K-slices are added through LDS in a fixed order,
-//     so a row of x gives the same bits whatever else is in the batch.
+//   * a wave owns 16 rows of W; W is the A operand of MFMA 16x16x32 (16 rows x
+//     32 k) and is read straight from memory in operand order, 64 contiguous
+//     bytes of a row per load instruction, the next loads issued before the
+//     products of the current ones;
+//   * the waves of a block own neighbouring rows and the same range of K, so
+//     they share x: the block stages x through LDS in pieces of 256 (or 128) columns
+//     (double-buffered, rows padded against bank conflicts) and every wave
+//     reads its B operands from there; up to four column sets of 16 rows of
+//     x share each read of W;
+//   * a matrix with few rows is also split along K over blocks (grid.y) so
+//     that every CU has work; each slice writes 32-bit partial sums and a
+//     second kernel adds the slices in a fixed order.  A row of x therefore
+//     gives the same bits whatever else is in the batch.
 //
 // The reference hands these products to cuBLASLt, with its own kernels for the
 // one-row case (v3/crates/rvllm-cutlass/src/cublaslt.rs:184-277, kernels/fp8_gemv.cu);
 // this is the bf16 counterpart of the latter for up to 64 rows.
+#include <stdlib.h>
+
 #include "common.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 sk_bf16x8;
@@ -28,24 +32,12 @@ union SkFrag {
   uint4 u4;
 };
 
-#define SK_MAX_WAVES 16
-
-template <typename TC>
-__device__ __forceinline__ void sk_store4(TC* p, float a, float b, float c, float d);
-template <>
-__device__ __forceinline__ void sk_store4<float>(float* p, float a, float b, float c, float d) {
-  p[0] = a;
-  p[1] = b;
-  p[2] = c;
-  p[3] = d;
-}
-template <>
-__device__ __forceinline__ void sk_store4<uint16_t>(uint16_t* p, float a, float b, float c, float d) {
-  p[0] = rv_f32_to_bf16_bits(a);
-  p[1] = rv_f32_to_bf16_bits(b);
-  p[2] = rv_f32_to_bf16_bits(c);
-  p[3] = rv_f32_to_bf16_bits(d);
-}
+// Columns of x staged at a time: 256, or 128 for more than 32 rows of x so that
+// the two buffers stay well inside LDS.  Rows are padded by 8 elements: the
+// row stride is then 4 banks off a multiple of 64 banks, and the 16 lanes that
+// read the same columns of 16 rows hit 64 different banks.
+#define SK_KC_OF(MT) ((MT) <= 2 ? 256 : 128)
+#define SK_MAX_WAVES 8
 
 template <typename TC>
 __device__ __forceinline__ void sk_store1(TC* p, float a);
@@ -58,127 +50,199 @@ __device__ __forceinline__ void sk_store1<uint16_t>(uint16_t* p, float a) {
   p[0] = rv_f32_to_bf16_bits(a);
 }
 
+// grid (row blocks, K slices); block = waves x 64.  With one slice the result
+// goes to `out` as TC; with more, slice s writes 32-bit sums to part[s][M][N].
 template <int MT, typename TC>
 __global__ void __launch_bounds__(SK_MAX_WAVES * 64)
-gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, TC* __restrict__ out, int M, int N,
-                   int K, long long ldx, long long ldw, long long ldc, int slice_len) {
-  extern __shared__ float red[];  // [waves][MT][64][4]
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, TC* __restrict__ out,
+                   float* __restrict__ part, int M, int N, int K, long long ldx, long long ldw, long long ldc,
+                   int slice_len) {
+  constexpr int SK_KC = SK_KC_OF(MT);
+  constexpr int SK_ROW = SK_KC + 8;
+  __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][SK_ROW];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   const int waves = blockDim.x >> 6;
   const int r16 = lane & 15;
   const int kb = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = (blockIdx.x * waves + wave) * 16;
+  const bool wave_has_rows = n0 < N;
   const int row = n0 + r16 < N ? n0 + r16 : N - 1;
-  const int kbeg = wave * slice_len;
+  const int kbeg = blockIdx.y * slice_len;
   const int kend = kbeg + slice_len < K ? kbeg + slice_len : K;
+  const int chunks = (kend - kbeg + SK_KC - 1) / SK_KC;
+
+  // staging: the block copies x[0 : MT*16, chunk] into LDS, 16 bytes a thread and turn
+  constexpr int PIECES = MT * 16 * (SK_KC / 8);  // 16-byte pieces in a chunk
+  // a thread holds at most PIECES / 256 pieces (blocks have at least 4 waves)
+  constexpr int MAX_REGS = (PIECES + 255) / 256;
+  uint4 staged[MAX_REGS];
+  auto stage_load = [&](int c) {
+#pragma unroll
+    for (int n = 0; n < MAX_REGS; ++n) {
+      const int p = tid + n * (int)blockDim.x;
+      const int m = p / (SK_KC / 8);
+      const int col = (p % (SK_KC / 8)) * 8;
+      const int k = kbeg + c * SK_KC + col;
+      staged[n] = (p < PIECES && m < M && k < kend) ? *(const uint4*)(x + (size_t)m * ldx + k)
+                                                   : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stage_store = [&](int buf) {
+#pragma unroll
+    for (int n = 0; n < MAX_REGS; ++n) {
+      const int p = tid + n * (int)blockDim.x;
+      if (p < PIECES) *(uint4*)(&xs[buf][p / (SK_KC / 8)][(p % (SK_KC / 8)) * 8]) = staged[n];
+    }
+  };
 
   sk_f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = (sk_f32x4){0.f, 0.f, 0.f, 0.f};
+  const uint16_t* wrow = w + (size_t)row * ldw + kbeg;
 
-  const uint16_t* wrow = w + (size_t)row * ldw;
-  const uint16_t* xrow[MT];
-  bool xok[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + r16;
-    xok[mt] = m < M;
-    xrow[mt] = x + (size_t)(xok[mt] ? m : 0) * ldx;
-  }
-
-  for (int k0 = kbeg; k0 < kend; k0 += 128) {
-    SkFrag a[4];
+  SkFrag a_cur[4], a_nxt[4];
+  auto load_w = [&](int koff, SkFrag* a) {  // koff: offset inside the slice of the 128 columns to read
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int off = k0 + kb * 32 + j * 8;
-      if (off < kend)
-        a[j].u4 = *(const uint4*)(wrow + off);
-      else
-        a[j].u4 = make_uint4(0, 0, 0, 0);
+      const int off = koff + j * 32 + kb * 8;
+      a[j].u4 = (wave_has_rows && kbeg + off < kend) ? *(const uint4*)(wrow + off) : make_uint4(0, 0, 0, 0);
     }
+  };
+  // The first read of W is issued before x is staged: the two latencies overlap.
+  load_w(0, a_cur);
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+
+  for (int c = 0; c < chunks; ++c) {
+    const int buf = c & 1;
+    if (c + 1 < chunks) stage_load(c + 1);  // in flight while this chunk is multiplied
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int off = k0 + kb * 32 + j * 8;
+    for (int it = 0; it < SK_KC / 128; ++it) {
+      const int koff = c * SK_KC + it * 128;
+      load_w(koff + 128, a_nxt);  // past the slice's end this reads nothing (zeros)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        SkFrag bfrag;
-        if (off < kend && xok[mt])
-          bfrag.u4 = *(const uint4*)(xrow[mt] + off);
-        else
-          bfrag.u4 = make_uint4(0, 0, 0, 0);
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].v, bfrag.v, acc[mt], 0, 0, 0);
+      for (int j = 0; j < 4; ++j) {
+        const int col = it * 128 + j * 32 + kb * 8;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          SkFrag b;
+          b.u4 = *(const uint4*)(&xs[buf][mt * 16 + r16][col]);
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[j].v, b.v, acc[mt], 0, 0, 0);
+        }
       }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a_cur[j] = a_nxt[j];
+    }
+    if (c + 1 < chunks) {
+      stage_store(buf ^ 1);  // the other buffer was last read in chunk c - 1, before the barrier below
+      __syncthreads();
     }
   }
 
-  if (waves > 1) {
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      float* dst = red + (((size_t)wave * MT + mt) * 64 + lane) * 4;
-      dst[0] = acc[mt][0];
-      dst[1] = acc[mt][1];
-      dst[2] = acc[mt][2];
-      dst[3] = acc[mt][3];
-    }
-    __syncthreads();
-    if (wave != 0) return;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-      for (int wv = 0; wv < waves; ++wv) {  // fixed order: the sum does not depend on timing
-        const float* src = red + (((size_t)wv * MT + mt) * 64 + lane) * 4;
-        s0 += src[0];
-        s1 += src[1];
-        s2 += src[2];
-        s3 += src[3];
-      }
-      acc[mt] = (sk_f32x4){s0, s1, s2, s3};
-    }
-  }
-  // a lane holds out[m = mt*16 + r16][n0 + kb*4 .. + 3]
+  if (!wave_has_rows) return;
+  // a lane holds the sums for x row m = mt*16 + r16 and W rows n0 + kb*4 .. + 3
   const int nb = n0 + kb * 4;
+  const bool sliced = gridDim.y > 1;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r16;
     if (m >= M) continue;
-    TC* o = out + (size_t)m * ldc + nb;
-    if (nb + 3 < N) {
-      sk_store4<TC>(o, acc[mt][0], acc[mt][1], acc[mt][2], acc[mt][3]);
+    if (sliced) {
+      float* o = part + ((size_t)blockIdx.y * M + m) * N + nb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (nb + i < N) o[i] = acc[mt][i];
     } else {
-      if (nb + 0 < N) sk_store1<TC>(o + 0, acc[mt][0]);
-      if (nb + 1 < N) sk_store1<TC>(o + 1, acc[mt][1]);
-      if (nb + 2 < N) sk_store1<TC>(o + 2, acc[mt][2]);
+      TC* o = out + (size_t)m * ldc + nb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (nb + i < N) sk_store1<TC>(o + i, acc[mt][i]);
     }
   }
 }
 
-// How many K-slices (waves a block) a product of this shape gets: enough that
-// about 2048 waves run, each slice a multiple of 128 long.
-extern "C" int rv_gemm_skinny_waves(int N, int K) {
+// out[m][n] = sum over slices of part[s][m][n], slices in order.
+template <typename TC>
+__global__ void sk_reduce_kernel(const float* __restrict__ part, TC* __restrict__ out, int slices, int M, int N,
+                                 long long ldc) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)M * N) return;
+  const int m = (int)(idx / N);
+  const int n = (int)(idx - (long long)m * N);
+  float s = 0.f;
+  for (int i = 0; i < slices; ++i) s += part[(size_t)i * M * N + idx];
+  sk_store1<TC>(out + (size_t)m * ldc + n, s);
+}
+
+// The plan for a shape: waves a block, K slices, columns a slice (a multiple of
+// 128).  The chip runs all blocks at once, a few per CU, so the time is set by
+// the CU with the most blocks: the plan looks for a number of blocks that
+// fills the CUs evenly (close below a multiple of their number), with about
+// 2048 waves in all and slices that are not too short.
+#define SK_NUM_CUS 256
+extern "C" void rv_gemm_skinny_plan(int N, int K, int* waves, int* slices, int* slice_len) {
   const int tiles = rv_div_up(N, 16);
-  int waves = rv_div_up(2048, tiles);
-  const int max_by_k = K / 128 > 0 ? K / 128 : 1;
-  if (waves > max_by_k) waves = max_by_k;
-  if (waves > SK_MAX_WAVES) waves = SK_MAX_WAVES;
-  if (waves < 1) waves = 1;
-  return waves;
+  const int units = rv_div_up(K, 128);
+  double best_time = 1e300;
+  int best_w = 4, best_len = units * 128, best_s = 1;
+  const double w_bytes = 2.0 * N * K;
+  for (int wv = 4; wv <= SK_MAX_WAVES; ++wv) {
+    const int row_blocks = rv_div_up(tiles, wv);
+    for (int per = units; per >= 1; --per) {  // 128-column units a slice
+      const int s = rv_div_up(units, per);
+      if (per * s - units >= per) continue;  // the last slice would be empty
+      // a model of the time, in bytes moved at full speed
+      const double part_bytes = s > 1 ? 2.0 * 4.0 * s * 16.0 * N : 0.0;  // partial sums written and read, 16 rows of x
+      const long long blocks = (long long)row_blocks * s;
+      const long long rounds = (blocks + SK_NUM_CUS - 1) / SK_NUM_CUS;
+      const double fill = (double)blocks / (double)(rounds * SK_NUM_CUS);  // evenness over the CUs
+      const double total_waves = (double)blocks * wv;
+      const double in_flight = total_waves >= 1024.0 ? 1.0 : total_waves / 1024.0;  // enough loads in flight
+      const double rows_used = (double)tiles / (double)(row_blocks * wv);            // waves without rows
+      const double startup = (per + 2.0) / per;  // a wave's start costs about two steps
+      const double time = (w_bytes + part_bytes) / (fill * in_flight * rows_used) * startup;
+      if (time < best_time * (1.0 - 1e-9)) {
+        best_time = time;
+        best_w = wv;
+        best_len = per * 128;
+        best_s = s;
+      }
+    }
+  }
+  *waves = best_w;
+  *slice_len = best_len;
+  *slices = best_s;
+}
+
+// Floats of workspace that rv_gemm_skinny needs for this shape (0 when unsliced).
+extern "C" long long rv_gemm_skinny_workspace(int M, int N, int K) {
+  int waves, slices, len;
+  rv_gemm_skinny_plan(N, K, &waves, &slices, &len);
+  return slices > 1 ? (long long)slices * M * N : 0;
 }
 
 template <int MT, typename TC>
-static int sk_launch(hipStream_t stream, const uint16_t* x, const uint16_t* w, TC* out, int M, int N, int K,
-                     long long ldx, long long ldw, long long ldc) {
-  const int waves = rv_gemm_skinny_waves(N, K);
-  const int slice_len = rv_div_up(rv_div_up(K, waves), 128) * 128;
-  const size_t lds = waves > 1 ? (size_t)waves * MT * 64 * 4 * sizeof(float) : 0;
-  gemm_skinny_kernel<MT, TC><<<dim3(rv_div_up(N, 16)), dim3(waves * 64), lds, stream>>>(x, w, out, M, N, K, ldx, ldw,
-                                                                                       ldc, slice_len);
+static int sk_launch(hipStream_t stream, const uint16_t* x, const uint16_t* w, TC* out, float* part, int M, int N,
+                     int K, long long ldx, long long ldw, long long ldc) {
+  int waves, slices, len;
+  rv_gemm_skinny_plan(N, K, &waves, &slices, &len);
+  if (slices > 1 && part == nullptr) return rv_fail("gemm_skinny: this shape needs a workspace");
+  dim3 grid(rv_div_up(rv_div_up(N, 16), waves), slices);
+  gemm_skinny_kernel<MT, TC><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc, len);
   RV_LAUNCH_CHECK("gemm_skinny");
+  if (slices > 1) {
+    const long long total = (long long)M * N;
+    sk_reduce_kernel<TC><<<dim3(rv_div_up(total, 256)), dim3(256), 0, stream>>>(part, out, slices, M, N, ldc);
+    RV_LAUNCH_CHECK("gemm_skinny_reduce");
+  }
   return 0;
 }
 
-extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, void* out, int out_dtype, int M, int N,
-                              int K, long long ldx, long long ldw, long long ldc) {
+extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, void* out, int out_dtype, float* part,
+                              int M, int N, int K, long long ldx, long long ldw, long long ldc) {
   RV_CHECK(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K and the row strides must be multiples of 8");
   RV_CHECK(ldx >= K && ldw >= K && ldc >= N, "gemm_skinny: leading dimensions too small");
@@ -187,11 +251,12 @@ extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, 
   const int mt = rv_div_up(M, 16);
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
-#define SK_CASE(MTV)                                                                                      \
-  case MTV:                                                                                               \
-    if (out_dtype == RV_F32) return sk_launch<MTV, float>(stream, xp, wp, (float*)out, M, N, K, ldx, ldw, ldc); \
-    if (out_dtype == RV_BF16)                                                                             \
-      return sk_launch<MTV, uint16_t>(stream, xp, wp, (uint16_t*)out, M, N, K, ldx, ldw, ldc);           \
+#define SK_CASE(MTV)                                                                                  \
+  case MTV:                                                                                           \
+    if (out_dtype == RV_F32)                                                                          \
+      return sk_launch<MTV, float>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc);        \
+    if (out_dtype == RV_BF16)                                                                         \
+      return sk_launch<MTV, uint16_t>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc);  \
     break;
   switch (mt) {
     SK_CASE(1)

@@ -9,6 +9,7 @@ trace replay all go through it.
 
 from __future__ import annotations
 
+import dataclasses
 import os
 from typing import Hashable, Optional, Sequence
 
@@ -58,6 +59,53 @@ class ModelRunner:
         width = -(-cfg.max_model_len // ps)
         self.builder = BatchBuilder(self.device, cfg.max_num_batched_tokens, cfg.max_num_seqs,
                                     {name: width for name in self.cache.groups})
+        # Captured decode steps, by (requests, context bucket).
+        self._graphs: dict[tuple[int, int], tuple] = {}
+        self._graph_pool = None
+        self.graph_replays = 0
+
+    # ---- decode steps from captured graphs -------------------------------
+    GRAPH_CONTEXT_BUCKET = 1024
+    GRAPH_MAX_REQUESTS = 64  # beyond this the products go to the library, which stays out of graphs
+
+    def _graph_key(self, batch: StepBatch):
+        """The key of the captured graph that can run this batch, or None.
+
+        A graph replays launches with fixed grids, so it covers steps of one
+        shape: B requests with one token each, logits wanted for all of them,
+        contexts up to a bucket's upper end (the attention kernel's split plan
+        is made for that end; splits past a request's own context are empty).
+        The reference captures its decode step the same way, once per batch
+        size (v3/crates/rvllm-runtime/src/gemma4_serve.rs:594-694)."""
+        if not (self.config.use_graphs and self.dtype == torch.bfloat16 and batch.decode_only):
+            return None
+        if batch.num_logit_rows != batch.num_tokens or batch.num_requests > self.GRAPH_MAX_REQUESTS:
+            return None
+        bucket = -(-batch.max_context // self.GRAPH_CONTEXT_BUCKET) * self.GRAPH_CONTEXT_BUCKET
+        return batch.num_requests, bucket
+
+    def _forward(self, batch: StepBatch) -> torch.Tensor:
+        key = self._graph_key(batch)
+        if key is None:
+            return self.model.forward(batch, self.storage.views)
+        entry = self._graphs.get(key)
+        if entry is None:
+            # The first step of a shape runs eagerly and is then recorded
+            # (recording runs nothing) for the steps that follow.
+            logits = self.model.forward(batch, self.storage.views)
+            shaped = dataclasses.replace(batch, max_context=key[1])
+            graph = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                static_logits = self.model.forward(shaped, self.storage.views)
+            if self._graph_pool is None:
+                self._graph_pool = graph.pool()
+            self._graphs[key] = (graph, static_logits)
+            return logits
+        graph, static_logits = entry
+        graph.replay()
+        self.graph_replays += 1
+        return static_logits
 
     # ---- construction --------------------------------------------------
     @classmethod
@@ -133,7 +181,7 @@ class ModelRunner:
             self.cache.extend(p.request, p.start + len(p.tokens))
         tables = {name: [self.cache.table(p.request, name) for p in portions] for name in self.cache.groups}
         batch = self.builder.build(portions, tables, [self.cache.slot(p.request) for p in portions])
-        logits = self.model.forward(batch, self.storage.views)
+        logits = self._forward(batch)
         for p in portions:
             self.cache.commit(p.request, p.start + len(p.tokens))
         return logits

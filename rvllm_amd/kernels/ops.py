@@ -387,11 +387,15 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optional[t
     ldx = x.stride(0) if m > 1 else k
     ldw = w.stride(0) if n > 1 else k
     ldc = out.stride(0) if m > 1 else n
+    lib.rv_gemm_skinny_workspace.restype = ctypes.c_longlong
+    floats = lib.rv_gemm_skinny_workspace(_c_int(min(m, SKINNY_MAX_ROWS)), _c_int(n), _c_int(k))
+    part = torch.empty(floats, dtype=torch.float32, device=x.device) if floats else None
     for m0 in range(0, m, SKINNY_MAX_ROWS):
         rows = min(SKINNY_MAX_ROWS, m - m0)
         _check(lib.rv_gemm_skinny(_stream(), ctypes.c_void_p(x.data_ptr() + m0 * ldx * 2), _ptr(w),
                                   ctypes.c_void_p(out.data_ptr() + m0 * ldc * out.element_size()), _dt(out),
-                                  _c_int(rows), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(ldc)))
+                                  _ptr(part), _c_int(rows), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw),
+                                  _c_ll(ldc)))
     return out
 
 

@@ -125,6 +125,44 @@ def test_requests_set_back_when_pages_run_out_give_the_same_tokens(model_dirs):
                                                            tight.runner.cache.groups.values()))
 
 
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_decode_steps_replayed_from_a_graph_match_eager_steps(model_dirs, plain_models, name):
+    """Every replay is checked, with eager work (prompts of new requests, a
+    request leaving) and synchronisations between the replays."""
+    weights, cfg = plain_models[name]
+    common = dict(dtype="bfloat16", max_model_len=256, max_num_seqs=4, max_num_batched_tokens=64,
+                  max_prefill_chunk=64, max_cache_tokens=1024)
+    eager = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(use_graphs=False, **common)).runner
+    graph = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(use_graphs=True, **common)).runner
+    seqs = tt.make_sequences(cfg["vocab"], [40, 75, 23], seed=8)
+    refs = {rid: plain_gemma.forward(weights, cfg, ids, torch.float64) for rid, ids in seqs.items()}
+    done = {rid: 0 for rid in seqs}
+    for runner in (eager, graph):
+        for rid, ids in seqs.items():
+            runner.add_request(rid)
+            runner.step([(rid, ids[:10], [])])  # prompts run eagerly
+    for rid in seqs:
+        done[rid] = 10
+    live = list(seqs)
+    for it in range(30):
+        if it == 12:  # one request leaves: another shape, another graph
+            for runner in (eager, graph):
+                runner.release("r2")
+            live.remove("r2")
+        entries = [(rid, [seqs[rid][done[rid]]], [0]) for rid in live if done[rid] < len(seqs[rid])]
+        if not entries:
+            break
+        a = eager.step(entries).float().cpu()
+        b = graph.step(entries).float().cpu()  # .cpu() synchronises between the replays
+        for row, (rid, _, _) in enumerate(entries):
+            tt.compare(b[row:row + 1].numpy(), refs[rid][done[rid]:done[rid] + 1], "bfloat16", f"replay {it} {rid}")
+            tt.compare(a[row:row + 1].numpy(), refs[rid][done[rid]:done[rid] + 1], "bfloat16", f"eager {it} {rid}")
+            done[rid] += 1
+        assert (a - b).abs().max() <= 1e-2 * a.abs().max(), f"replay {it} differs from the eager step"
+    assert graph.graph_replays >= 20 and eager.graph_replays == 0
+    assert len(graph._graphs) >= 2
+
+
 def test_eos_and_capacity_reasons(model_dirs):
     engine = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(dtype="float32", max_model_len=128,
                                                                     max_num_seqs=2, max_cache_tokens=32))
