@@ -269,8 +269,9 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
 
 MFMA_ATTENTION_MAX_HEAD_DIM = 256
 MFMA_ATTENTION_MAX_GROUP = 16
-# Waves that fill the chip: 256 CUs, 4 SIMDs each, two waves a SIMD.
-_ATTENTION_TARGET_UNITS = 2048
+# Units (waves) a launch aims for: the kernel runs one wave a SIMD, 1024 at once on 256 CUs; a few more
+# even out units of different length.
+_ATTENTION_TARGET_UNITS = 1536
 
 
 def mfma_attention_covers(k_pages: torch.Tensor, v_pages: torch.Tensor, num_q_heads: int) -> bool:
