@@ -66,34 +66,153 @@ extern "C" int rv_embed_gather(hipStream_t stream, const void* table, int table_
 }
 
 // ---------------------------------------------------------------------------
-// RMSNorm: y = x * rsqrt(mean(x^2) + eps) * (offset + w)
-// One block per row.
+// Row kernels keep a row in registers: one block per row, a thread owns E
+// groups of V consecutive elements (V = 16 bytes' worth when the width allows,
+// else 1), so a row is read once and written once whatever the number of
+// passes over it.
 // ---------------------------------------------------------------------------
+#define ROW_MAX_E 16
+
 template <typename T>
+struct RowVec {
+  static constexpr int V = 16 / sizeof(T);
+};
+
+template <typename T, int V>
+__device__ __forceinline__ void row_load(const T* p, float* out) {
+  if constexpr (V == 1) {
+    out[0] = rv_to_float(p[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    const float4 v = *(const float4*)p;
+    out[0] = v.x, out[1] = v.y, out[2] = v.z, out[3] = v.w;
+  } else {
+    const uint4 v = *(const uint4*)p;
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      out[2 * i] = __uint_as_float(u[i] << 16);
+      out[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+    }
+  }
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void row_store(T* p, const float* in) {
+  if constexpr (V == 1) {
+    p[0] = rv_from_float<T>(in[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    *(float4*)p = make_float4(in[0], in[1], in[2], in[3]);
+  } else {
+    uint32_t u[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      u[i] = (uint32_t)rv_f32_to_bf16_bits(in[2 * i]) | ((uint32_t)rv_f32_to_bf16_bits(in[2 * i + 1]) << 16);
+    *(uint4*)p = make_uint4(u[0], u[1], u[2], u[3]);
+  }
+}
+
+// V weights starting at element i; the weight vector may be float or bf16.
+template <int V>
+__device__ __forceinline__ void row_load_w(const void* w, int w_f32, int i, float* out) {
+  if (w_f32) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) out[v] = ((const float*)w)[i + v];
+  } else {
+#pragma unroll
+    for (int v = 0; v < V; ++v) out[v] = rv_to_float(((const bf16_t*)w)[i + v]);
+  }
+}
+
+// V values of a branch starting at element i of row `row`: either stored as T,
+// or as the sum of `slices` 32-bit partial sums (the K slices of a product),
+// added in the order of the slices.
+template <typename T, int V>
+__device__ __forceinline__ void row_load_branch(const void* branch, int slices, long long slice_stride, size_t at,
+                                                float* out) {
+  if (slices == 0) {
+    row_load<T, V>((const T*)branch + at, out);
+  } else {
+#pragma unroll
+    for (int v = 0; v < V; ++v) out[v] = 0.f;
+    for (int s = 0; s < slices; ++s) {
+      const float* p = (const float*)branch + (size_t)s * slice_stride + at;
+      if constexpr (V >= 4) {
+#pragma unroll
+        for (int v = 0; v < V; v += 4) {
+          const float4 q = *(const float4*)(p + v);
+          out[v] += q.x, out[v + 1] += q.y, out[v + 2] += q.z, out[v + 3] += q.w;
+        }
+      } else {
+        out[0] += p[0];
+      }
+    }
+  }
+}
+
+static void row_geometry(int width, int v, int* block, int* e) {
+  const int groups = rv_div_up(width, v);
+  int b = rv_div_up(groups, 64) * 64;
+  if (b > 1024) b = 1024;
+  *block = b;
+  *e = rv_div_up(groups, b);
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm: y = x * rsqrt(mean(x^2) + eps) * (offset + w)
+// ---------------------------------------------------------------------------
+template <typename T, int V, int E>
 __global__ void rmsnorm_kernel(const T* __restrict__ x, const int* __restrict__ row_index, const void* __restrict__ w,
                                int w_f32, T* __restrict__ y, int width, float eps, float offset) {
   __shared__ float scratch[16];
   const int in_row = row_index ? row_index[blockIdx.x] : (int)blockIdx.x;
   const T* xr = x + (size_t)in_row * width;
   T* yr = y + (size_t)blockIdx.x * width;
+  float val[E][V];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = rv_to_float(xr[i]);
-    ss += v * v;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = (e * blockDim.x + threadIdx.x) * V;
+    if (i < width) {
+      row_load<T, V>(xr + i, val[e]);
+#pragma unroll
+      for (int v = 0; v < V; ++v) ss += val[e][v] * val[e][v];
+    }
   }
   ss = rv_block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = rv_to_float(xr[i]);
-    yr[i] = rv_from_float<T>(v * inv * (offset + rv_load_w(w, w_f32, i)));
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = (e * blockDim.x + threadIdx.x) * V;
+    if (i < width) {
+      float g[V];
+      row_load_w<V>(w, w_f32, i, g);
+#pragma unroll
+      for (int v = 0; v < V; ++v) val[e][v] = val[e][v] * inv * (offset + g[v]);
+      row_store<T, V>(yr + i, val[e]);
+    }
   }
 }
 
-static int norm_block(int width) {
-  int b = 64;
-  while (b < width / 4 && b < 1024) b *= 2;  // about four elements a thread
-  return b;
-}
+// Picks the instantiation for a width: vectors when the width is a multiple of
+// 16 bytes' worth of elements, and as many groups a thread as the width needs.
+#define ROW_DISPATCH(KERNEL, T, width, grid, stream, ...)                                               \
+  do {                                                                                                  \
+    constexpr int VV = RowVec<T>::V;                                                                    \
+    int block_, e_;                                                                                     \
+    if ((width) % VV == 0) {                                                                            \
+      row_geometry(width, VV, &block_, &e_);                                                            \
+      if (e_ <= 1) KERNEL<T, VV, 1><<<grid, dim3(block_), 0, stream>>>(__VA_ARGS__);                    \
+      else if (e_ <= 2) KERNEL<T, VV, 2><<<grid, dim3(block_), 0, stream>>>(__VA_ARGS__);               \
+      else if (e_ <= 4) KERNEL<T, VV, 4><<<grid, dim3(block_), 0, stream>>>(__VA_ARGS__);               \
+      else return rv_fail("row kernel: width %d is too large", width);                                  \
+    } else {                                                                                            \
+      row_geometry(width, 1, &block_, &e_);                                                             \
+      if (e_ <= 1) KERNEL<T, 1, 1><<<grid, dim3(block_), 0, stream>>>(__VA_ARGS__);                     \
+      else if (e_ <= 4) KERNEL<T, 1, 4><<<grid, dim3(block_), 0, stream>>>(__VA_ARGS__);                \
+      else if (e_ <= ROW_MAX_E) KERNEL<T, 1, ROW_MAX_E><<<grid, dim3(block_), 0, stream>>>(__VA_ARGS__); \
+      else return rv_fail("row kernel: width %d is too large", width);                                  \
+    }                                                                                                   \
+  } while (0)
 
 // Output row r is the norm of input row row_index[r] (of row r when row_index
 // is null); the caller guarantees the indices are inside x.
@@ -101,13 +220,13 @@ extern "C" int rv_rmsnorm(hipStream_t stream, const void* x, const int* row_inde
                           int dtype, int rows, int width, float eps, float offset) {
   RV_CHECK(rows >= 0 && width > 0, "rmsnorm: bad sizes rows=%d width=%d", rows, width);
   if (rows == 0) return 0;
-  dim3 grid(rows), block(norm_block(width));
+  dim3 grid(rows);
   if (dtype == RV_F32)
-    rmsnorm_kernel<float><<<grid, block, 0, stream>>>((const float*)x, row_index, w, w_f32, (float*)y, width, eps,
-                                                      offset);
+    ROW_DISPATCH(rmsnorm_kernel, float, width, grid, stream, (const float*)x, row_index, w, w_f32, (float*)y, width,
+                 eps, offset);
   else if (dtype == RV_BF16)
-    rmsnorm_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, row_index, w, w_f32, (bf16_t*)y, width, eps,
-                                                       offset);
+    ROW_DISPATCH(rmsnorm_kernel, bf16_t, width, grid, stream, (const bf16_t*)x, row_index, w, w_f32, (bf16_t*)y,
+                 width, eps, offset);
   else
     return rv_fail("rmsnorm: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("rmsnorm");
@@ -117,57 +236,81 @@ extern "C" int rv_rmsnorm(hipStream_t stream, const void* x, const int* row_inde
 // ---------------------------------------------------------------------------
 // residual += RMSNorm(branch; w_post); optionally next = RMSNorm(residual; w_next)
 // The normed branch is added in 32-bit and the sum rounded once; the second
-// norm sees the residual as it is stored (rounded to T).
+// norm sees the residual as it is stored (rounded to T).  The branch is either
+// stored as T or given as `slices` 32-bit partial sums of a product.
 // ---------------------------------------------------------------------------
-template <typename T>
-__global__ void add_rmsnorm_kernel(const T* __restrict__ branch, const void* __restrict__ w_post, int w_post_f32,
-                                   T* __restrict__ residual, const void* __restrict__ w_next, int w_next_f32,
-                                   T* __restrict__ next, int width, float eps, float offset, float eps_next,
-                                   float offset_next) {
+template <typename T, int V, int E>
+__global__ void add_rmsnorm_kernel(const void* __restrict__ branch, int slices, long long slice_stride,
+                                   const void* __restrict__ w_post, int w_post_f32, T* __restrict__ residual,
+                                   const void* __restrict__ w_next, int w_next_f32, T* __restrict__ next, int width,
+                                   float eps, float offset, float eps_next, float offset_next) {
   __shared__ float scratch[16];
-  const T* br = branch + (size_t)blockIdx.x * width;
-  T* rr = residual + (size_t)blockIdx.x * width;
+  const size_t row0 = (size_t)blockIdx.x * width;
+  T* rr = residual + row0;
+  float val[E][V];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = rv_to_float(br[i]);
-    ss += v * v;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = (e * blockDim.x + threadIdx.x) * V;
+    if (i < width) {
+      row_load_branch<T, V>(branch, slices, slice_stride, row0 + i, val[e]);
+#pragma unroll
+      for (int v = 0; v < V; ++v) ss += val[e][v] * val[e][v];
+    }
   }
   ss = rv_block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
   float ss2 = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float n = rv_to_float(br[i]) * inv * (offset + rv_load_w(w_post, w_post_f32, i));
-    const T stored = rv_from_float<T>(rv_to_float(rr[i]) + n);
-    rr[i] = stored;
-    const float r = rv_to_float(stored);
-    ss2 += r * r;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = (e * blockDim.x + threadIdx.x) * V;
+    if (i < width) {
+      float g[V], r[V];
+      row_load_w<V>(w_post, w_post_f32, i, g);
+      row_load<T, V>(rr + i, r);
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        // the residual as it reads back after the store
+        val[e][v] = rv_round_to<T>(r[v] + val[e][v] * inv * (offset + g[v]));
+        ss2 += val[e][v] * val[e][v];
+      }
+      row_store<T, V>(rr + i, val[e]);
+    }
   }
   if (next == nullptr) return;
   ss2 = rv_block_sum(ss2, scratch);
   const float inv2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
-  T* nr = next + (size_t)blockIdx.x * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    // each thread re-reads only what it wrote itself
-    const float r = rv_to_float(rr[i]);
-    nr[i] = rv_from_float<T>(r * inv2 * (offset_next + rv_load_w(w_next, w_next_f32, i)));
+  T* nr = next + row0;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = (e * blockDim.x + threadIdx.x) * V;
+    if (i < width) {
+      float g[V];
+      row_load_w<V>(w_next, w_next_f32, i, g);
+#pragma unroll
+      for (int v = 0; v < V; ++v) val[e][v] = val[e][v] * inv2 * (offset_next + g[v]);
+      row_store<T, V>(nr + i, val[e]);
+    }
   }
 }
 
-extern "C" int rv_add_rmsnorm(hipStream_t stream, const void* branch, const void* w_post, int w_post_f32,
-                              void* residual, const void* w_next, int w_next_f32, void* next, int dtype, int rows,
-                              int width, float eps, float offset, float eps_next, float offset_next) {
+// `slices` 0: branch holds T values [rows, width].  Otherwise branch holds
+// 32-bit partial sums [slices][rows][width] (slice_stride elements apart).
+extern "C" int rv_add_rmsnorm(hipStream_t stream, const void* branch, int slices, long long slice_stride,
+                              const void* w_post, int w_post_f32, void* residual, const void* w_next, int w_next_f32,
+                              void* next, int dtype, int rows, int width, float eps, float offset, float eps_next,
+                              float offset_next) {
   RV_CHECK(rows >= 0 && width > 0, "add_rmsnorm: bad sizes rows=%d width=%d", rows, width);
   RV_CHECK((w_next == nullptr) == (next == nullptr), "add_rmsnorm: next norm needs both weight and output");
+  RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= (long long)rows * width), "add_rmsnorm: bad partial sums");
   if (rows == 0) return 0;
-  dim3 grid(rows), block(norm_block(width));
+  dim3 grid(rows);
   if (dtype == RV_F32)
-    add_rmsnorm_kernel<float><<<grid, block, 0, stream>>>((const float*)branch, w_post, w_post_f32, (float*)residual,
-                                                          w_next, w_next_f32, (float*)next, width, eps, offset,
-                                                          eps_next, offset_next);
+    ROW_DISPATCH(add_rmsnorm_kernel, float, width, grid, stream, branch, slices, slice_stride, w_post, w_post_f32,
+                 (float*)residual, w_next, w_next_f32, (float*)next, width, eps, offset, eps_next, offset_next);
   else if (dtype == RV_BF16)
-    add_rmsnorm_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)branch, w_post, w_post_f32,
-                                                           (bf16_t*)residual, w_next, w_next_f32, (bf16_t*)next, width,
-                                                           eps, offset, eps_next, offset_next);
+    ROW_DISPATCH(add_rmsnorm_kernel, bf16_t, width, grid, stream, branch, slices, slice_stride, w_post, w_post_f32,
+                 (bf16_t*)residual, w_next, w_next_f32, (bf16_t*)next, width, eps, offset, eps_next, offset_next);
   else
     return rv_fail("add_rmsnorm: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("add_rmsnorm");
@@ -183,31 +326,50 @@ __device__ __forceinline__ float rv_gelu_tanh(float z) {
 }
 __device__ __forceinline__ float rv_silu(float z) { return z / (1.0f + expf(-z)); }
 
-template <typename T, int ACT>
-__global__ void gated_act_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, long long total) {
-  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= total) return;
-  const long long t = idx / inter;
-  const int i = (int)(idx - t * inter);
-  const T* row = gu + t * 2 * (long long)inter;
-  const float g = rv_to_float(row[i]);
-  const float u = rv_to_float(row[inter + i]);
-  const float a = ACT == 0 ? rv_gelu_tanh(g) : rv_silu(g);
-  out[idx] = rv_from_float<T>(a * u);
+template <typename T, int V, int ACT>
+__global__ void gated_act_kernel(const void* __restrict__ gu, int slices, long long slice_stride, T* __restrict__ out,
+                                 int inter, long long groups_total) {
+  const long long gidx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gidx >= groups_total) return;
+  const int groups_per_row = inter / V;
+  const long long t = gidx / groups_per_row;
+  const int i = (int)(gidx - t * groups_per_row) * V;
+  const size_t at = (size_t)t * 2 * inter + i;
+  float g[V], u[V];
+  row_load_branch<T, V>(gu, slices, slice_stride, at, g);
+  row_load_branch<T, V>(gu, slices, slice_stride, at + inter, u);
+#pragma unroll
+  for (int v = 0; v < V; ++v) g[v] = (ACT == 0 ? rv_gelu_tanh(g[v]) : rv_silu(g[v])) * u[v];
+  row_store<T, V>(out + (size_t)t * inter + i, g);
 }
 
-extern "C" int rv_gated_act(hipStream_t stream, const void* gu, void* out, int dtype, int rows, int inter, int act) {
+// `slices` 0: gu holds T values [rows, 2*inter]; otherwise 32-bit partial sums
+// [slices][rows][2*inter], slice_stride elements apart.
+extern "C" int rv_gated_act(hipStream_t stream, const void* gu, int slices, long long slice_stride, void* out,
+                            int dtype, int rows, int inter, int act) {
   RV_CHECK(rows >= 0 && inter > 0, "gated_act: bad sizes rows=%d inter=%d", rows, inter);
   RV_CHECK(act == 0 || act == 1, "gated_act: unknown activation %d", act);
+  RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= 2ll * rows * inter), "gated_act: bad partial sums");
   if (rows == 0) return 0;
-  const long long total = (long long)rows * inter;
-  dim3 grid(rv_div_up(total, 256)), block(256);
-#define RV_GA(T, A) gated_act_kernel<T, A><<<grid, block, 0, stream>>>((const T*)gu, (T*)out, inter, total)
-  if (dtype == RV_F32 && act == 0) RV_GA(float, 0);
-  else if (dtype == RV_F32 && act == 1) RV_GA(float, 1);
-  else if (dtype == RV_BF16 && act == 0) RV_GA(bf16_t, 0);
-  else if (dtype == RV_BF16 && act == 1) RV_GA(bf16_t, 1);
+#define RV_GA(T, V, A)                                                                                       \
+  do {                                                                                                       \
+    const long long groups = (long long)rows * (inter / V);                                                  \
+    gated_act_kernel<T, V, A><<<dim3(rv_div_up(groups, 256)), dim3(256), 0, stream>>>(gu, slices, slice_stride, \
+                                                                                     (T*)out, inter, groups); \
+  } while (0)
+#define RV_GA_T(T)                                     \
+  do {                                                 \
+    constexpr int VV = RowVec<T>::V;                   \
+    if (inter % VV == 0) {                             \
+      if (act == 0) RV_GA(T, VV, 0); else RV_GA(T, VV, 1); \
+    } else {                                           \
+      if (act == 0) RV_GA(T, 1, 0); else RV_GA(T, 1, 1);   \
+    }                                                  \
+  } while (0)
+  if (dtype == RV_F32) RV_GA_T(float);
+  else if (dtype == RV_BF16) RV_GA_T(bf16_t);
   else return rv_fail("gated_act: unsupported dtype %d", dtype);
+#undef RV_GA_T
 #undef RV_GA
   RV_LAUNCH_CHECK("gated_act");
   return 0;

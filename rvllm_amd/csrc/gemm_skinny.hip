@@ -224,16 +224,23 @@ extern "C" long long rv_gemm_skinny_workspace(int M, int N, int K) {
   return slices > 1 ? (long long)slices * M * N : 0;
 }
 
+// Number of K slices of this shape (1 = unsliced).
+extern "C" int rv_gemm_skinny_slices(int N, int K) {
+  int waves, slices, len;
+  rv_gemm_skinny_plan(N, K, &waves, &slices, &len);
+  return slices;
+}
+
 template <int MT, typename TC>
 static int sk_launch(hipStream_t stream, const uint16_t* x, const uint16_t* w, TC* out, float* part, int M, int N,
-                     int K, long long ldx, long long ldw, long long ldc) {
+                     int K, long long ldx, long long ldw, long long ldc, int do_reduce) {
   int waves, slices, len;
   rv_gemm_skinny_plan(N, K, &waves, &slices, &len);
   if (slices > 1 && part == nullptr) return rv_fail("gemm_skinny: this shape needs a workspace");
   dim3 grid(rv_div_up(rv_div_up(N, 16), waves), slices);
   gemm_skinny_kernel<MT, TC><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc, len);
   RV_LAUNCH_CHECK("gemm_skinny");
-  if (slices > 1) {
+  if (slices > 1 && do_reduce) {
     const long long total = (long long)M * N;
     sk_reduce_kernel<TC><<<dim3(rv_div_up(total, 256)), dim3(256), 0, stream>>>(part, out, slices, M, N, ldc);
     RV_LAUNCH_CHECK("gemm_skinny_reduce");
@@ -241,8 +248,11 @@ static int sk_launch(hipStream_t stream, const uint16_t* x, const uint16_t* w, T
   return 0;
 }
 
+// With `do_reduce` 0 a sliced product leaves its 32-bit partial sums in `part`
+// ([slices][M][N]) for a consumer that adds them itself, and `out` is not
+// written; an unsliced product always writes `out`.
 extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, void* out, int out_dtype, float* part,
-                              int M, int N, int K, long long ldx, long long ldw, long long ldc) {
+                              int M, int N, int K, long long ldx, long long ldw, long long ldc, int do_reduce) {
   RV_CHECK(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K and the row strides must be multiples of 8");
   RV_CHECK(ldx >= K && ldw >= K && ldc >= N, "gemm_skinny: leading dimensions too small");
@@ -254,9 +264,9 @@ extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, 
 #define SK_CASE(MTV)                                                                                  \
   case MTV:                                                                                           \
     if (out_dtype == RV_F32)                                                                          \
-      return sk_launch<MTV, float>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc);        \
+      return sk_launch<MTV, float>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc, do_reduce);        \
     if (out_dtype == RV_BF16)                                                                         \
-      return sk_launch<MTV, uint16_t>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc);  \
+      return sk_launch<MTV, uint16_t>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc, do_reduce);  \
     break;
   switch (mt) {
     SK_CASE(1)
@@ -266,4 +276,21 @@ extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, 
   }
 #undef SK_CASE
   return rv_fail("gemm_skinny: unsupported output dtype %d", out_dtype);
+}
+
+// out[m][n] (bf16 or 32-bit) = sum over slices of part[s][m][n].
+extern "C" int rv_reduce_slices(hipStream_t stream, const float* part, void* out, int out_dtype, int slices, int M,
+                                int N) {
+  RV_CHECK(slices >= 1 && M >= 0 && N > 0 && part && out, "reduce_slices: bad arguments");
+  if (M == 0) return 0;
+  const long long total = (long long)M * N;
+  if (out_dtype == RV_F32)
+    sk_reduce_kernel<float><<<dim3(rv_div_up(total, 256)), dim3(256), 0, stream>>>(part, (float*)out, slices, M, N, N);
+  else if (out_dtype == RV_BF16)
+    sk_reduce_kernel<uint16_t><<<dim3(rv_div_up(total, 256)), dim3(256), 0, stream>>>(part, (uint16_t*)out, slices, M,
+                                                                                    N, N);
+  else
+    return rv_fail("reduce_slices: unsupported output dtype %d", out_dtype);
+  RV_LAUNCH_CHECK("reduce_slices");
+  return 0;
 }

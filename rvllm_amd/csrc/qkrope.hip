@@ -20,8 +20,19 @@
 
 #define QKR_MAX_HD 512
 
+// One value of the projection's output: stored as T, or the sum of `slices`
+// 32-bit partial sums (the K slices of the product), added in their order.
 template <typename T>
-__global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
+__device__ __forceinline__ float qkr_input(const void* qkv, int slices, long long slice_stride, size_t at) {
+  if (slices == 0) return rv_to_float(((const T*)qkv)[at]);
+  float sum = 0.f;
+  for (int s = 0; s < slices; ++s) sum += ((const float*)qkv)[(size_t)s * slice_stride + at];
+  return sum;
+}
+
+template <typename T>
+__global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int slices, long long slice_stride,
+                                             T* __restrict__ q_out,
                                              const void* __restrict__ q_w, const void* __restrict__ k_w, int w_f32,
                                              float eps, float offset, const float* __restrict__ inv_freq, int rot,
                                              const int* __restrict__ positions, const int* __restrict__ token_req,
@@ -36,7 +47,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
   const int total_heads = nq + 2 * nkv;
   if (head >= total_heads) return;  // whole wave leaves together; no block barrier below
 
-  const T* src = qkv + (size_t)t * total_heads * hd + (size_t)head * hd;
+  const size_t src = (size_t)t * total_heads * hd + (size_t)head * hd;  // first element of this head in qkv
   const bool is_q = head < nq;
   const bool is_k = !is_q && head < nq + nkv;
   const int pos = positions[t];
@@ -57,7 +68,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
     } else {
       // values are stored as projected, transposed inside the page
       T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
-      for (int d = lane; d < hd; d += RV_WAVE) col[(size_t)d * page_size] = src[d];
+      for (int d = lane; d < hd; d += RV_WAVE)
+        col[(size_t)d * page_size] = rv_from_float<T>(qkr_input<T>(qkv, slices, slice_stride, src + d));
       return;
     }
   }
@@ -66,7 +78,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
   const void* w = is_q ? q_w : k_w;
   float ss = 0.f;
   for (int d = lane; d < hd; d += RV_WAVE) {
-    const float v = rv_to_float(src[d]);
+    const float v = qkr_input<T>(qkv, slices, slice_stride, src + d);
     x[d] = v;
     ss += v * v;
   }
@@ -98,12 +110,17 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
   }
 }
 
-extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, void* q_out, const void* q_w,
+// `slices` 0: qkv holds T values [tokens, (nq + 2 nkv) * hd]; otherwise 32-bit
+// partial sums [slices][tokens][...], slice_stride elements apart.
+extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int slices, long long slice_stride,
+                                        void* q_out, const void* q_w,
                                         const void* k_w, int w_f32, float eps, float offset, const float* inv_freq,
                                         int rot, const int* positions, const int* token_req, const int* block_table,
                                         int table_width, void* k_pages, void* v_pages, int page_size, int num_pages,
                                         int dtype, int num_tokens, int nq, int nkv, int hd, int write_kv) {
   RV_CHECK(num_tokens >= 0 && nq > 0 && nkv > 0, "qk_norm_rope: bad sizes T=%d nq=%d nkv=%d", num_tokens, nq, nkv);
+  RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= (long long)num_tokens * (nq + 2 * nkv) * hd),
+           "qk_norm_rope: bad partial sums");
   RV_CHECK(hd >= 2 && hd % 2 == 0 && hd <= QKR_MAX_HD, "qk_norm_rope: head_dim %d must be even and <= %d", hd,
            QKR_MAX_HD);
   RV_CHECK(rot >= 0 && rot <= hd && rot % 2 == 0, "qk_norm_rope: rotary_dim %d must be even and <= head_dim %d", rot, hd);
@@ -115,11 +132,11 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, voi
   dim3 grid(num_tokens, rv_div_up(nq + 2 * nkv, 4)), block(4 * RV_WAVE);
   if (dtype == RV_F32)
     qk_norm_rope_kv_write_kernel<float><<<grid, block, 0, stream>>>(
-        (const float*)qkv, (float*)q_out, q_w, k_w, w_f32, eps, offset, inv_freq, rot, positions, token_req,
+        qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, inv_freq, rot, positions, token_req,
         block_table, table_width, (float*)k_pages, (float*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv);
   else if (dtype == RV_BF16)
     qk_norm_rope_kv_write_kernel<bf16_t><<<grid, block, 0, stream>>>(
-        (const bf16_t*)qkv, (bf16_t*)q_out, q_w, k_w, w_f32, eps, offset, inv_freq, rot, positions, token_req,
+        qkv, slices, slice_stride, (bf16_t*)q_out, q_w, k_w, w_f32, eps, offset, inv_freq, rot, positions, token_req,
         block_table, table_width, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv);
   else
     return rv_fail("qk_norm_rope: unsupported dtype %d", dtype);

@@ -100,6 +100,48 @@ def _cache_geometry(k_pages: torch.Tensor, v_pages: torch.Tensor, what: str) -> 
     return num_pages, nkv, page_size, hd
 
 
+class SlicedSums:
+    """The result of a product whose K range was split over blocks, not yet
+    added up: 32-bit partial sums ``[slices, rows, width]``.  The kernels that
+    consume a product's result (norm + residual add, q/k norm and rotation,
+    gated activation) add the slices themselves, in their order, which saves a
+    kernel and a rounding; anything else calls ``as_tensor``."""
+
+    def __init__(self, data: torch.Tensor, dtype: torch.dtype):
+        self.data = data  # [slices, rows, width] float32
+        self.dtype = dtype  # what the product's result would be stored as
+        self.slices, self.rows, self.width = data.shape
+
+    @property
+    def shape(self):
+        return (self.rows, self.width)
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def as_tensor(self) -> torch.Tensor:
+        out = torch.empty((self.rows, self.width), dtype=self.dtype, device=self.data.device)
+        _check(library().rv_reduce_slices(_stream(), _ptr(self.data), _ptr(out), _dt(out), _c_int(self.slices),
+                                          _c_int(self.rows), _c_int(self.width)))
+        return out
+
+
+def as_tensor(x) -> torch.Tensor:
+    """A plain tensor from a tensor or from unreduced ``SlicedSums``."""
+    return x.as_tensor() if isinstance(x, SlicedSums) else x
+
+
+def _branch_args(x, what: str):
+    """(pointer, slices, slice stride, rows, width, dtype) of a kernel input
+    that is a tensor or ``SlicedSums``."""
+    if isinstance(x, SlicedSums):
+        return _ptr(x.data), x.slices, x.rows * x.width, x.rows, x.width, x.dtype
+    _gpu(x)
+    _need(x.dim() == 2, f"{what}: a matrix is expected")
+    return _ptr(x), 0, 0, x.shape[0], x.shape[1], x.dtype
+
+
 # --------------------------------------------------------------------------
 def embed_gather(table: torch.Tensor, ids: torch.Tensor, scale: float, out: torch.Tensor) -> torch.Tensor:
     _gpu(table, ids, out)
@@ -137,14 +179,14 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float,
     return out
 
 
-def add_rmsnorm(branch: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, residual: torch.Tensor,
+def add_rmsnorm(branch, weight: torch.Tensor, eps: float, offset: float, residual: torch.Tensor,
                 next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0, next_offset: float = 0.0,
                 next_out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-    """residual += rmsnorm(branch); with ``next_weight`` also returns rmsnorm(residual)."""
-    _gpu(branch, weight, residual, next_weight, next_out)
-    width = branch.shape[-1]
-    rows = branch.numel() // width
-    _need(residual.shape == branch.shape and residual.dtype == branch.dtype, "add_rmsnorm: residual must match branch")
+    """residual += rmsnorm(branch); with ``next_weight`` also returns rmsnorm(residual).
+    ``branch`` is a tensor or ``SlicedSums``."""
+    bptr, slices, stride, rows, width, bdtype = _branch_args(branch, "add_rmsnorm")
+    _gpu(weight, residual, next_weight, next_out)
+    _need(residual.shape == (rows, width) and residual.dtype == bdtype, "add_rmsnorm: residual must match branch")
     _need(weight.shape == (width,), "add_rmsnorm: bad weight shape")
     if next_weight is not None:
         _need(next_weight.shape == (width,), "add_rmsnorm: bad next weight shape")
@@ -152,9 +194,9 @@ def add_rmsnorm(branch: torch.Tensor, weight: torch.Tensor, eps: float, offset: 
             next_out = torch.empty_like(residual)
         _need(next_out.shape == residual.shape and next_out.dtype == residual.dtype, "add_rmsnorm: bad next_out")
     _check(library().rv_add_rmsnorm(
-        _stream(), _ptr(branch), _ptr(weight), _c_int(weight.dtype == torch.float32), _ptr(residual),
-        _ptr(next_weight), _c_int(next_weight is not None and next_weight.dtype == torch.float32),
-        _ptr(next_out if next_weight is not None else None), _dt(branch), _c_int(rows), _c_int(width), _c_float(eps),
+        _stream(), bptr, _c_int(slices), _c_ll(stride), _ptr(weight), _c_int(weight.dtype == torch.float32),
+        _ptr(residual), _ptr(next_weight), _c_int(next_weight is not None and next_weight.dtype == torch.float32),
+        _ptr(next_out if next_weight is not None else None), _dt(residual), _c_int(rows), _c_int(width), _c_float(eps),
         _c_float(offset), _c_float(next_eps), _c_float(next_offset)))
     return next_out if next_weight is not None else None
 
@@ -162,18 +204,18 @@ def add_rmsnorm(branch: torch.Tensor, weight: torch.Tensor, eps: float, offset: 
 ACTIVATIONS = {"gelu_pytorch_tanh": 0, "gelu_tanh": 0, "silu": 1}
 
 
-def gated_act(gate_up: torch.Tensor, activation: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]"""
-    _gpu(gate_up, out)
-    rows, two_i = gate_up.shape
+def gated_act(gate_up, activation: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]; ``gate_up`` is a tensor or ``SlicedSums``."""
+    gptr, slices, stride, rows, two_i, dtype = _branch_args(gate_up, "gated_act")
     _need(two_i % 2 == 0, "gated_act: width must be even")
     inter = two_i // 2
     if out is None:
-        out = torch.empty((rows, inter), dtype=gate_up.dtype, device=gate_up.device)
-    _need(out.shape == (rows, inter) and out.dtype == gate_up.dtype, "gated_act: bad out")
+        out = torch.empty((rows, inter), dtype=dtype, device=gate_up.device)
+    _gpu(out)
+    _need(out.shape == (rows, inter) and out.dtype == dtype, "gated_act: bad out")
     _need(activation in ACTIVATIONS, f"gated_act: unknown activation {activation!r}")
-    _check(library().rv_gated_act(_stream(), _ptr(gate_up), _ptr(out), _dt(gate_up), _c_int(rows), _c_int(inter),
-                                  _c_int(ACTIVATIONS[activation])))
+    _check(library().rv_gated_act(_stream(), gptr, _c_int(slices), _c_ll(stride), _ptr(out), _dt(out), _c_int(rows),
+                                  _c_int(inter), _c_int(ACTIVATIONS[activation])))
     return out
 
 
@@ -199,17 +241,17 @@ def gemm_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Ten
     return out
 
 
-def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Optional[torch.Tensor],
+def qk_norm_rope_kv_write(qkv, q_out: torch.Tensor, q_weight: Optional[torch.Tensor],
                           k_weight: Optional[torch.Tensor], eps: float, offset: float,
                           inv_freq: Optional[torch.Tensor], rotary_dim: int, positions: torch.Tensor,
                           token_req: torch.Tensor, block_table: Optional[torch.Tensor],
                           k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], num_q_heads: int,
                           num_kv_heads: int, head_dim: int, write_kv: bool = True) -> torch.Tensor:
-    _gpu(qkv, q_out, q_weight, k_weight, inv_freq, positions, token_req, block_table, k_pages, v_pages)
+    qptr, slices, stride, n, qkv_width, qkv_dtype = _branch_args(qkv, "qk_norm_rope")
+    _gpu(q_out, q_weight, k_weight, inv_freq, positions, token_req, block_table, k_pages, v_pages)
     _i32(positions, token_req)
-    n = qkv.shape[0]
-    _need(qkv.shape == (n, (num_q_heads + 2 * num_kv_heads) * head_dim), "qk_norm_rope: bad qkv shape")
-    _need(q_out.shape == (n, num_q_heads * head_dim) and q_out.dtype == qkv.dtype, "qk_norm_rope: bad q_out")
+    _need(qkv_width == (num_q_heads + 2 * num_kv_heads) * head_dim, "qk_norm_rope: bad qkv shape")
+    _need(q_out.shape == (n, num_q_heads * head_dim) and q_out.dtype == qkv_dtype, "qk_norm_rope: bad q_out")
     _need(positions.numel() >= n and token_req.numel() >= n, "qk_norm_rope: positions/token_req too short")
     w_f32 = 0
     if q_weight is not None:
@@ -225,13 +267,14 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _i32(block_table)
         num_pages, nkv, page_size, hd = _cache_geometry(k_pages, v_pages, "qk_norm_rope")
         _need((nkv, hd) == (num_kv_heads, head_dim), "qk_norm_rope: cache pages do not fit the heads")
-        _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "qk_norm_rope: cache dtype differs")
+        _need(k_pages.dtype == qkv_dtype and v_pages.dtype == qkv_dtype, "qk_norm_rope: cache dtype differs")
         width = block_table.shape[1]
     _check(library().rv_qk_norm_rope_kv_write(
-        _stream(), _ptr(qkv), _ptr(q_out), _ptr(q_weight), _ptr(k_weight), _c_int(w_f32), _c_float(eps),
+        _stream(), qptr, _c_int(slices), _c_ll(stride), _ptr(q_out), _ptr(q_weight), _ptr(k_weight), _c_int(w_f32),
+        _c_float(eps),
         _c_float(offset), _ptr(inv_freq), _c_int(rotary_dim if inv_freq is not None else 0), _ptr(positions),
         _ptr(token_req), _ptr(block_table), _c_int(width), _ptr(k_pages), _ptr(v_pages), _c_int(page_size),
-        _c_int(num_pages), _dt(qkv), _c_int(n), _c_int(num_q_heads), _c_int(num_kv_heads), _c_int(head_dim),
+        _c_int(num_pages), _dt(q_out), _c_int(n), _c_int(num_q_heads), _c_int(num_kv_heads), _c_int(head_dim),
         _c_int(int(write_kv))))
     return q_out
 
@@ -366,37 +409,47 @@ def topk_select(logits: torch.Tensor, k: int, inv_temp: torch.Tensor) -> tuple[t
     return vals, idx
 
 
-def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optional[torch.Tensor]:
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+              out_dtype: Optional[torch.dtype] = None, sliced_ok: bool = False):
     """out = x @ w^T on the matrix cores for bf16 inputs; None when no
     hand-written kernel covers the shape (the caller then uses another path).
 
     Products with up to 64 rows run the kernel that is built around reading
     ``w`` once.  A 32-bit result of more rows (logits at many positions) runs
     it over blocks of 64 rows; a bf16 result of more rows is left to the
-    library product."""
+    library product.  With ``sliced_ok`` a product whose K range is split over
+    blocks returns its partial sums as ``SlicedSums`` instead of adding them."""
     m, k = x.shape
     n = w.shape[0]
-    if k % 8 or x.stride(1) != 1 or w.stride(1) != 1 or out.stride(1) != 1:
+    out_dtype = out.dtype if out is not None else (out_dtype or x.dtype)
+    if k % 8 or x.stride(1) != 1 or w.stride(1) != 1 or (out is not None and out.stride(1) != 1):
         return None
     if (m > 1 and x.stride(0) % 8) or (n > 1 and w.stride(0) % 8) or x.data_ptr() % 16 or w.data_ptr() % 16:
         return None
-    if m > SKINNY_MAX_ROWS and out.dtype != torch.float32:
+    if m > SKINNY_MAX_ROWS and out_dtype != torch.float32:
         return None
-    _need(x.is_cuda and w.is_cuda and out.is_cuda, "gemm: arguments must live on the GPU")
-    _need(out.shape == (m, n) and w.shape[1] == k, "gemm: shapes do not fit")
+    _need(x.is_cuda and w.is_cuda, "gemm: arguments must live on the GPU")
+    _need(w.shape[1] == k and (out is None or out.shape == (m, n)), "gemm: shapes do not fit")
     lib = library()
     ldx = x.stride(0) if m > 1 else k
     ldw = w.stride(0) if n > 1 else k
+    slices = lib.rv_gemm_skinny_slices(_c_int(n), _c_int(k))
+    if sliced_ok and out is None and slices > 1 and m <= SKINNY_MAX_ROWS:
+        part = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+        _check(lib.rv_gemm_skinny(_stream(), _ptr(x), _ptr(w), None, _dt(x), _ptr(part), _c_int(m), _c_int(n),
+                                  _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(n), _c_int(0)))
+        return SlicedSums(part, out_dtype)
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     ldc = out.stride(0) if m > 1 else n
-    lib.rv_gemm_skinny_workspace.restype = ctypes.c_longlong
-    floats = lib.rv_gemm_skinny_workspace(_c_int(min(m, SKINNY_MAX_ROWS)), _c_int(n), _c_int(k))
-    part = torch.empty(floats, dtype=torch.float32, device=x.device) if floats else None
+    rows_max = min(m, SKINNY_MAX_ROWS)
+    part = torch.empty(slices * rows_max * n, dtype=torch.float32, device=x.device) if slices > 1 else None
     for m0 in range(0, m, SKINNY_MAX_ROWS):
         rows = min(SKINNY_MAX_ROWS, m - m0)
         _check(lib.rv_gemm_skinny(_stream(), ctypes.c_void_p(x.data_ptr() + m0 * ldx * 2), _ptr(w),
                                   ctypes.c_void_p(out.data_ptr() + m0 * ldc * out.element_size()), _dt(out),
                                   _ptr(part), _c_int(rows), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw),
-                                  _c_ll(ldc)))
+                                  _c_ll(ldc), _c_int(1)))
     return out
 
 

@@ -76,7 +76,7 @@ class PagedAttention(Mixer):
     # ---- run ---------------------------------------------------------
     def forward(self, x: torch.Tensor, step, cache: KVCacheView) -> torch.Tensor:
         n = x.shape[0]
-        qkv = linear(x, self.w_qkv)
+        qkv = linear(x, self.w_qkv, sliced_ok=True)
         q = torch.empty((n, self.q_size), dtype=x.dtype, device=x.device)
         table = step.block_tables[cache.group]
         norm = self.qk_norm or {}
@@ -88,7 +88,7 @@ class PagedAttention(Mixer):
         attn = torch.empty_like(q)
         ops.paged_attention(q, cache.k_pages, cache.v_pages, table, step, attn, self.num_heads, self.scale,
                             self.window)
-        return linear(attn, self.w_o)
+        return linear(attn, self.w_o, sliced_ok=True)
 
 
 MIXERS.register("attention", PagedAttention)

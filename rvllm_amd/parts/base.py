@@ -127,7 +127,9 @@ class Norm(Part):
         """residual += norm(branch), in place; when ``then`` is given also
         return then(residual).  The default runs the pieces one by one; a norm
         with a fused kernel overrides it."""
-        normed = self.forward(branch)
+        from ..kernels import ops
+
+        normed = self.forward(ops.as_tensor(branch))
         residual.add_(normed)
         return then.forward(residual, out=then_out) if then is not None else None
 
@@ -144,7 +146,9 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    """Mixes information between the tokens of a request."""
+    """Mixes information between the tokens of a request.  ``forward`` returns
+    ``[tokens, hidden]``: a tensor, or ``ops.SlicedSums`` when its last product
+    was left unreduced for the norm that follows (``ops.as_tensor`` reduces)."""
 
     def cache_need(self):
         return None

@@ -41,9 +41,9 @@ class GatedMLP(FeedForward):
         self.w_down = tensors[f"{p}.down_proj.weight"].to(device=device, dtype=dtype).contiguous()
 
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
-        gate_up = linear(x, self.w_gate_up)
+        gate_up = linear(x, self.w_gate_up, sliced_ok=True)
         act = ops.gated_act(gate_up, self.activation)
-        return linear(act, self.w_down)
+        return linear(act, self.w_down, sliced_ok=True)
 
 
 FEED_FORWARDS.register("gated_mlp", GatedMLP)

@@ -18,10 +18,16 @@ from ..kernels import ops
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
-           out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+           out_dtype: Optional[torch.dtype] = None, sliced_ok: bool = False):
+    """``sliced_ok``: the caller hands the result to a kernel that takes
+    ``ops.SlicedSums`` (the unreduced K slices of a product with few rows)."""
     m, k = x.shape
     n = w.shape[0]
     out_dtype = out_dtype or (out.dtype if out is not None else x.dtype)
+    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and m > 0:
+        fast = ops.gemm_bf16(x, w, out, out_dtype=out_dtype, sliced_ok=sliced_ok)
+        if fast is not None:
+            return fast
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     if m == 0:
@@ -31,9 +37,6 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
             raise ops.KernelError(f"linear: unsupported weight dtype {w.dtype}")
         return ops.gemm_plain(x, w, out)
     if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-        fast = ops.gemm_bf16(x, w, out)
-        if fast is not None:
-            return fast
         if out.dtype == torch.bfloat16:
             return torch.matmul(x, w.t(), out=out)
         return ops.gemm_plain(x, w, out)

@@ -455,3 +455,46 @@ def test_kernels_refuse_what_they_cannot_do():
                                   None, None, None, 1, 1, hd, write_kv=False)
     with pytest.raises(ops.KernelError, match="k="):
         ops.topk_select(dev(torch.randn(1, 5000)), 2000, dev(torch.ones(1)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_consumers_add_up_the_slices_of_a_product(dtype):
+    """A product with few rows may hand its K slices to the next kernel
+    unreduced; each consumer gives what it gives for the reduced tensor."""
+    g = torch.Generator().manual_seed(30)
+    slices, rows, width = 5, 7, 96
+    part = torch.randn(slices, rows, width, generator=g)
+    sums = ops.SlicedSums(dev(part), dtype)
+    whole = part.sum(0)
+    assert torch.allclose(sums.as_tensor().cpu().float(), whole, **tol(dtype))
+    reduced = dev(whole.to(dtype)) if dtype == torch.float32 else None
+    # norm + residual add
+    w = (torch.randn(width, generator=g) * 0.1).to(dtype)
+    res = torch.randn(rows, width, generator=g).to(dtype)
+    r1 = dev(res.clone())
+    ops.add_rmsnorm(sums, dev(w), 1e-6, 1.0, r1)
+    want = res.double() + P.rmsnorm(whole.double(), w.double(), 1e-6)
+    assert torch.allclose(r1.cpu().float(), want.float(), **tol(dtype))
+    # gated activation
+    act = ops.gated_act(sums, "gelu_pytorch_tanh").cpu().float()
+    want = F.gelu(whole[:, :48].double(), approximate="tanh") * whole[:, 48:].double()
+    assert torch.allclose(act, want.float(), **tol(dtype))
+    # q/k norm and rotation: 2 query heads, 2 kv heads of 16
+    q_out = torch.empty(rows, 32, dtype=dtype, device=DEV)
+    ops.qk_norm_rope_kv_write(sums, q_out, None, None, 0.0, 0.0, None, 0, dev(torch.arange(rows, dtype=torch.int32)),
+                              dev(torch.zeros(rows, dtype=torch.int32)), None, None, None, 2, 2, 16, write_kv=False)
+    assert torch.allclose(q_out.cpu().float(), whole[:, :32], **tol(dtype))
+    if dtype == torch.float32:  # in 32-bit the sliced and the reduced input give the same bits
+        r2 = dev(res.clone())
+        ops.add_rmsnorm(reduced, dev(w), 1e-6, 1.0, r2)
+        assert torch.equal(r1, r2)
+
+
+def test_sliced_product_through_the_skinny_kernel():
+    g = torch.Generator().manual_seed(31)
+    x, w = torch.randn(8, 2048, generator=g).bfloat16(), (torch.randn(2560, 2048, generator=g) * 0.05).bfloat16()
+    got = ops.gemm_bf16(dev(x), dev(w), sliced_ok=True)
+    assert isinstance(got, ops.SlicedSums) and got.slices > 1 and got.shape == (8, 2560)
+    want = x.double() @ w.double().T
+    assert torch.allclose(got.as_tensor().cpu().double(), want, atol=3e-2, rtol=2e-2)
+    assert torch.allclose(got.data.sum(0).cpu().double(), want, atol=1e-3, rtol=1e-4)

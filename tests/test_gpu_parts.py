@@ -15,6 +15,7 @@ from rvllm_amd.cache.storage import CacheStorage
 from rvllm_amd.config.engine_config import EngineConfig
 from rvllm_amd.engine.batch import BatchBuilder, Portion
 from rvllm_amd.engine.runner import ModelRunner
+from rvllm_amd.kernels import ops
 from rvllm_amd.models import Architecture, register_architecture, unregister_architecture
 from rvllm_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, LayerSpec, Mixer, ModelSpec,
                              ParamSpec, PartSpec, ScheduleEntry, StateNeed)
@@ -63,7 +64,7 @@ def test_feed_forward_part(dtype):
     want = P.feed_forward(x.double(), w["L.mlp.gate_proj.weight"], w["L.mlp.up_proj.weight"],
                           w["L.mlp.down_proj.weight"])
     tol = 1e-5 if dtype == torch.float32 else 2e-2
-    got = ff.forward(x.to(DEV), None).cpu().double()
+    got = ops.as_tensor(ff.forward(x.to(DEV), None)).cpu().double()
     assert (got - want).abs().max() <= tol * max(1.0, want.abs().max().item())
 
 
@@ -83,7 +84,8 @@ def run_portions(mixer, x, cuts):
     for n in cuts:
         cache.extend("r", start + n)
         batch = builder.build([Portion("r", [0] * n, start)], {group: [cache.table("r", group)]}, [cache.slot("r")])
-        outs.append(mixer.forward(x[start:start + n].to(DEV), batch, storage.views[0]).cpu())
+        # a part may hand back the unreduced K slices of its last product; as_tensor adds them up
+        outs.append(ops.as_tensor(mixer.forward(x[start:start + n].to(DEV), batch, storage.views[0])).cpu())
         cache.commit("r", start + n)
         start += n
     return torch.cat(outs)
