@@ -126,26 +126,46 @@ __device__ __forceinline__ void row_load_w(const void* w, int w_f32, int i, floa
 // V values of a branch starting at element i of row `row`: either stored as T,
 // or as the sum of `slices` 32-bit partial sums (the K slices of a product),
 // added in the order of the slices.
+template <int V>
+__device__ __forceinline__ void row_load_f32(const float* p, float* out) {
+  if constexpr (V >= 4) {
+#pragma unroll
+    for (int v = 0; v < V; v += 4) {
+      const float4 q = *(const float4*)(p + v);
+      out[v] = q.x, out[v + 1] = q.y, out[v + 2] = q.z, out[v + 3] = q.w;
+    }
+  } else {
+    out[0] = p[0];
+  }
+}
+
 template <typename T, int V>
 __device__ __forceinline__ void row_load_branch(const void* branch, int slices, long long slice_stride, size_t at,
                                                 float* out) {
   if (slices == 0) {
     row_load<T, V>((const T*)branch + at, out);
-  } else {
+    return;
+  }
 #pragma unroll
-    for (int v = 0; v < V; ++v) out[v] = 0.f;
-    for (int s = 0; s < slices; ++s) {
-      const float* p = (const float*)branch + (size_t)s * slice_stride + at;
-      if constexpr (V >= 4) {
+  for (int v = 0; v < V; ++v) out[v] = 0.f;
+  const float* p = (const float*)branch + at;
+  int s = 0;
+  // four slices are read at a time, so that their loads are in flight together;
+  // they are added in the order of the slices all the same
+  for (; s + 4 <= slices; s += 4) {
+    float q[4][V];
 #pragma unroll
-        for (int v = 0; v < V; v += 4) {
-          const float4 q = *(const float4*)(p + v);
-          out[v] += q.x, out[v + 1] += q.y, out[v + 2] += q.z, out[v + 3] += q.w;
-        }
-      } else {
-        out[0] += p[0];
-      }
-    }
+    for (int j = 0; j < 4; ++j) row_load_f32<V>(p + (size_t)(s + j) * slice_stride, q[j]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < V; ++v) out[v] += q[j][v];
+  }
+  for (; s < slices; ++s) {
+    float q[V];
+    row_load_f32<V>(p + (size_t)s * slice_stride, q);
+#pragma unroll
+    for (int v = 0; v < V; ++v) out[v] += q[v];
   }
 }
 

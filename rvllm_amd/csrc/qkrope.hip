@@ -25,8 +25,15 @@
 template <typename T>
 __device__ __forceinline__ float qkr_input(const void* qkv, int slices, long long slice_stride, size_t at) {
   if (slices == 0) return rv_to_float(((const T*)qkv)[at]);
+  const float* p = (const float*)qkv + at;
   float sum = 0.f;
-  for (int s = 0; s < slices; ++s) sum += ((const float*)qkv)[(size_t)s * slice_stride + at];
+  int s = 0;
+  for (; s + 4 <= slices; s += 4) {  // four loads in flight, added in the order of the slices
+    const float a = p[(size_t)s * slice_stride], b = p[(size_t)(s + 1) * slice_stride];
+    const float c = p[(size_t)(s + 2) * slice_stride], d = p[(size_t)(s + 3) * slice_stride];
+    sum = (((sum + a) + b) + c) + d;
+  }
+  for (; s < slices; ++s) sum += p[(size_t)s * slice_stride];
   return sum;
 }
 
