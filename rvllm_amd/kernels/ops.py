@@ -344,11 +344,18 @@ def plan_attention_splits(num_requests: int, max_portion: int, max_context: int,
     return tiles, -(-span // split_len), split_len
 
 
+# Portions of at least this many tokens go to the kernel whose blocks share key
+# tiles through LDS; shorter ones (decoded tokens above all) to the kernel that
+# splits a request's keys over many waves.
+PREFILL_MIN_PORTION = 16
+
+
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                          step, out: torch.Tensor, num_q_heads: int, scale: float, window: Optional[int],
-                         splits: Optional[tuple[int, int]] = None) -> torch.Tensor:
+                         splits: Optional[tuple[int, int]] = None, prefill_kernel: Optional[bool] = None) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``splits`` = (number, keys per
-    split) overrides the plan (tests use it to force every path)."""
+    split) overrides the plan and ``prefill_kernel`` the choice of kernel
+    (tests use them to force every path)."""
     _gpu(q, k_pages, v_pages, block_table, out)
     _i32(block_table)
     n = q.shape[0]
@@ -362,23 +369,57 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
           "attention (matrix cores): bad q or out shape")
     _need(n == step.num_tokens, "attention (matrix cores): q must hold the step's tokens")
     group = num_q_heads // nkv
-    tiles, num_splits, split_len = plan_attention_splits(step.num_requests, step.max_portion, step.max_context, nkv,
-                                                         group, window)
-    if splits is not None:
-        num_splits, split_len = splits
-        need = -(-step.max_context // 32) * 32
-        _need(window is not None or num_splits * split_len >= need, "attention: the splits do not cover the context")
-    part_o = part_ml = None
-    if num_splits > 1:
-        units = step.num_requests * tiles * nkv * num_splits
-        part_o = torch.empty(units * 16 * hd, dtype=torch.float32, device=q.device)
-        part_ml = torch.empty(units * 32, dtype=torch.float32, device=q.device)
-    entry = getattr(library(), f"rv_attn_mfma_g{(hd // 16 - 1) // 4}")
-    _check(entry(_stream(), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _c_int(block_table.shape[1]),
-                 _ptr(step.q_start), _ptr(step.chunk_start), _ptr(step.token_req), _ptr(out), _ptr(part_o),
-                 _ptr(part_ml), _c_int(n), _c_int(step.num_requests), _c_int(tiles), _c_int(num_q_heads), _c_int(nkv),
-                 _c_int(hd), _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_int(num_splits),
-                 _c_int(split_len), _c_float(scale)))
+    group_pad = 1
+    while group_pad < group:
+        group_pad *= 2
+    lib = library()
+    suffix = f"g{(hd // 16 - 1) // 4}"
+
+    # which requests go to which kernel
+    longest = step.max_portion
+    if prefill_kernel is None:
+        use_prefill = longest >= PREFILL_MIN_PORTION
+        portion_min = PREFILL_MIN_PORTION
+    else:
+        use_prefill, portion_min = prefill_kernel, 1
+    shortest_rest = 0  # longest portion left to the split-key kernel
+    if use_prefill and portion_min > 1:
+        starts = getattr(step, "host_q_start", None)
+        if starts is None:
+            starts = step.q_start.cpu().numpy()
+        lengths = [int(starts[i + 1] - starts[i]) for i in range(step.num_requests)]
+        shortest_rest = max([x for x in lengths if x < portion_min], default=0)
+    elif not use_prefill:
+        shortest_rest = longest
+
+    if use_prefill:
+        tokens_per_block = 64 // group_pad
+        tiles = -(-longest // tokens_per_block)
+        entry = getattr(lib, f"rv_attn_prefill_{suffix}")
+        _check(entry(_stream(), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+                     _c_int(block_table.shape[1]), _ptr(step.q_start), _ptr(step.chunk_start), _ptr(out), _c_int(n),
+                     _c_int(step.num_requests), _c_int(tiles), _c_int(num_q_heads), _c_int(nkv), _c_int(hd),
+                     _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_int(portion_min), _c_float(scale)))
+    if shortest_rest > 0:
+        tiles, num_splits, split_len = plan_attention_splits(step.num_requests, shortest_rest, step.max_context, nkv,
+                                                             group, window)
+        if splits is not None:
+            num_splits, split_len = splits
+            need = -(-step.max_context // 32) * 32
+            _need(window is not None or num_splits * split_len >= need,
+                  "attention: the splits do not cover the context")
+        part_o = part_ml = None
+        if num_splits > 1:
+            units = step.num_requests * tiles * nkv * num_splits
+            part_o = torch.empty(units * 16 * hd, dtype=torch.float32, device=q.device)
+            part_ml = torch.empty(units * 32, dtype=torch.float32, device=q.device)
+        entry = getattr(lib, f"rv_attn_mfma_{suffix}")
+        _check(entry(_stream(), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+                     _c_int(block_table.shape[1]), _ptr(step.q_start), _ptr(step.chunk_start), _ptr(step.token_req),
+                     _ptr(out), _ptr(part_o), _ptr(part_ml), _c_int(n), _c_int(step.num_requests), _c_int(tiles),
+                     _c_int(num_q_heads), _c_int(nkv), _c_int(hd), _c_int(page_size), _c_int(num_pages),
+                     _c_int(window or 0), _c_int(num_splits), _c_int(split_len),
+                     _c_int(portion_min - 1 if use_prefill else 0), _c_float(scale)))
     return out
 
 

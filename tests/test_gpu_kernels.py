@@ -301,7 +301,7 @@ class Case:
             num_tokens=T, num_requests=B, positions=dev(self.positions), token_req=dev(self.token_req),
             q_start=dev(torch.tensor(starts, dtype=torch.int32)),
             chunk_start=dev(torch.tensor([s for s, _ in portions], dtype=torch.int32)),
-            max_portion=max(n for _, n in portions), max_context=max(lengths))
+            max_portion=max(n for _, n in portions), max_context=max(lengths), host_q_start=starts)
 
     def reference(self, scale):
         outs = []
@@ -342,10 +342,25 @@ def test_paged_attention_generic(dtype, nq, nkv, hd, window):
                                        (5, 5, 240), (12, 4, 64)])
 @pytest.mark.parametrize("window", [None, 7, 100])
 @pytest.mark.parametrize("page_size", [16, 64])
-def test_paged_attention_mfma(nq, nkv, hd, window, page_size):
+@pytest.mark.parametrize("kernels", ["both", "split", "shared"])
+def test_paged_attention_mfma(nq, nkv, hd, window, page_size, kernels):
+    """``both``: as the engine runs a mixed batch, long portions through the
+    kernel that shares key tiles in LDS, short ones through the one that
+    splits keys; ``split`` / ``shared``: every request through one of them."""
     case = Case(MIXED, nq, nkv, hd, page_size, torch.bfloat16, 9, window)
     want = case.reference(hd ** -0.5).float()
-    assert torch.allclose(case.run("mfma", hd ** -0.5).float(), want, **tol(torch.bfloat16))
+    kw = {"both": {}, "split": {"prefill_kernel": False}, "shared": {"prefill_kernel": True}}[kernels]
+    assert torch.allclose(case.run("mfma", hd ** -0.5, **kw).float(), want, **tol(torch.bfloat16))
+
+
+def test_paged_attention_shared_tiles_long_prompt_portions():
+    """Portions as a scheduler cuts a long prompt: from position 0, continuing
+    at an odd position, and one that passes a window's edge."""
+    for portions, window in (([(0, 300)], None), ([(257, 130), (0, 70)], None), ([(0, 300)], 64), ([(990, 100)], 1024),
+                             ([(100, 257)], 100)):
+        case = Case(portions, 8, 4, 256, 16, torch.bfloat16, 13, window)
+        want = case.reference(1.0 / 16).float()
+        assert torch.allclose(case.run("mfma", 1.0 / 16).float(), want, **tol(torch.bfloat16)), (portions, window)
 
 
 @pytest.mark.parametrize("splits", [(1, 224), (2, 128), (7, 32), (4, 64)])
@@ -355,7 +370,8 @@ def test_paged_attention_mfma_every_split(splits, window):
     for some tiles: all give the same result."""
     case = Case(MIXED, 8, 4, 256, 16, torch.bfloat16, 10, window)
     want = case.reference(1.0 / 16).float()
-    assert torch.allclose(case.run("mfma", 1.0 / 16, splits=splits).float(), want, **tol(torch.bfloat16))
+    got = case.run("mfma", 1.0 / 16, splits=splits, prefill_kernel=False)
+    assert torch.allclose(got.float(), want, **tol(torch.bfloat16))
 
 
 def test_paged_attention_mfma_long_decode_batch():
