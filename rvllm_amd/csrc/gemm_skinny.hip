@@ -5,10 +5,10 @@
 //
 //   * a wave owns 16 rows of W; W is the A operand of MFMA 16x16x32 (16 rows x
 //     32 k) and is read straight from memory in operand order, 64 contiguous
-//     bytes of a row per load instruction, the next loads issued before the
-//     products of the current ones;
+//     bytes of a row per load instruction, several steps ahead of the products
+//     that use them;
 //   * the waves of a block own neighbouring rows and the same range of K, so
-//     they share x: the block stages x through LDS in pieces of 256 (or 128) columns
+//     they share x: the block stages x through LDS in pieces of 512 (or 256) columns
 //     (double-buffered, rows padded against bank conflicts) and every wave
 //     reads its B operands from there; up to four column sets of 16 rows of
 //     x share each read of W;
@@ -32,11 +32,19 @@ union SkFrag {
   uint4 u4;
 };
 
-// Columns of x staged at a time: 256, or 128 for more than 32 rows of x so that
-// the two buffers stay well inside LDS.  Rows are padded by 8 elements: the
-// row stride is then 4 banks off a multiple of 64 banks, and the 16 lanes that
+// A wave keeps SK_DEPTH steps of 128 columns of W in flight (a ring of
+// fragment sets in registers): with a memory latency of a few microseconds and
+// a step worth 4 KB a wave, that is what it takes for some 1024 waves to draw
+// the full bandwidth, and it lets a short slice issue all of its loads at once.
+// x is staged one ring's worth of columns at a time (SK_DEPTH * 128), two
+// buffers; for more than 32 rows of x the ring is shorter so that the buffers
+// stay inside LDS.  Rows of the staged x are padded by 8 elements: the row
+// stride is then 4 banks off a multiple of 64 banks, and the 16 lanes that
 // read the same columns of 16 rows hit 64 different banks.
-#define SK_KC_OF(MT) ((MT) <= 2 ? 256 : 128)
+#define SK_DEPTH_OF(MT) ((MT) <= 2 ? 4 : 2)
+// Waits until at most n of this wave's reads from memory are still in flight.
+// Reads come back in the order they were issued, so "all but the newest n".
+#define RV_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(0x3F70 | ((n) & 15) | ((((n) >> 4) & 3) << 14))
 #define SK_MAX_WAVES 8
 
 template <typename TC>
@@ -57,7 +65,8 @@ __global__ void __launch_bounds__(SK_MAX_WAVES * 64)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, TC* __restrict__ out,
                    float* __restrict__ part, int M, int N, int K, long long ldx, long long ldw, long long ldc,
                    int slice_len) {
-  constexpr int SK_KC = SK_KC_OF(MT);
+  constexpr int DEPTH = SK_DEPTH_OF(MT);
+  constexpr int SK_KC = DEPTH * 128;
   constexpr int SK_ROW = SK_KC + 8;
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][SK_ROW];
   const int tid = threadIdx.x;
@@ -73,27 +82,46 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   const int kend = kbeg + slice_len < K ? kbeg + slice_len : K;
   const int chunks = (kend - kbeg + SK_KC - 1) / SK_KC;
 
+  // Every read from memory below is unconditional, from an address clamped
+  // into the operand: a read under a branch makes the compiler wait for all
+  // earlier reads before the next product, which would undo the ring.  What a
+  // clamped read brings in is thrown away (x) or meets zeros of x (W).
+
   // staging: the block copies x[0 : MT*16, chunk] into LDS, 16 bytes a thread and turn
   constexpr int PIECES = MT * 16 * (SK_KC / 8);  // 16-byte pieces in a chunk
   // a thread holds at most PIECES / 256 pieces (blocks have at least 4 waves)
   constexpr int MAX_REGS = (PIECES + 255) / 256;
   uint4 staged[MAX_REGS];
+  const int last_k = kend - 8;  // the last 16-byte piece of this slice (slices are multiples of 8 long)
   auto stage_load = [&](int c) {
 #pragma unroll
     for (int n = 0; n < MAX_REGS; ++n) {
-      const int p = tid + n * (int)blockDim.x;
-      const int m = p / (SK_KC / 8);
-      const int col = (p % (SK_KC / 8)) * 8;
-      const int k = kbeg + c * SK_KC + col;
-      staged[n] = (p < PIECES && m < M && k < kend) ? *(const uint4*)(x + (size_t)m * ldx + k)
-                                                   : make_uint4(0, 0, 0, 0);
+      int p = tid + n * (int)blockDim.x;
+      p = p < PIECES ? p : PIECES - 1;
+      int m = p / (SK_KC / 8);
+      int k = kbeg + c * SK_KC + (p % (SK_KC / 8)) * 8;
+      m = m < M ? m : M - 1;
+      k = k < last_k ? k : last_k;
+      staged[n] = *(const uint4*)(x + (size_t)m * ldx + k);
     }
   };
-  auto stage_store = [&](int buf) {
+  auto stage_store = [&](int c, int buf) {
 #pragma unroll
     for (int n = 0; n < MAX_REGS; ++n) {
-      const int p = tid + n * (int)blockDim.x;
-      if (p < PIECES) *(uint4*)(&xs[buf][p / (SK_KC / 8)][(p % (SK_KC / 8)) * 8]) = staged[n];
+      int p = tid + n * (int)blockDim.x;
+      p = p < PIECES ? p : PIECES - 1;  // threads past the end repeat the last piece: the same bytes to the same place
+      const int m = p / (SK_KC / 8);
+      const int col = (p % (SK_KC / 8)) * 8;
+      // Columns past the slice's end become zeros, by a mask and not by a choice
+      // (a choice would let the compiler put the read under a branch again).
+      // Rows past M repeat row M - 1; their sums are never stored.
+      const unsigned keep = 0u - (unsigned)(kbeg + c * SK_KC + col < kend);
+      uint4 v = staged[n];
+      // The staged values count as used only from here on: otherwise the masking
+      // drifts up between the products, and its wait for x drains the ring.
+      asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+      v.x &= keep, v.y &= keep, v.z &= keep, v.w &= keep;
+      *(uint4*)(&xs[buf][m][col]) = v;
     }
   };
 
@@ -101,46 +129,52 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = (sk_f32x4){0.f, 0.f, 0.f, 0.f};
   const uint16_t* wrow = w + (size_t)row * ldw + kbeg;
+  const int last_off = kend - 8 - kbeg;
 
-  SkFrag a_cur[4], a_nxt[4];
+  SkFrag ring[DEPTH][4];
   auto load_w = [&](int koff, SkFrag* a) {  // koff: offset inside the slice of the 128 columns to read
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int off = koff + j * 32 + kb * 8;
-      a[j].u4 = (wave_has_rows && kbeg + off < kend) ? *(const uint4*)(wrow + off) : make_uint4(0, 0, 0, 0);
+      a[j].u4 = *(const uint4*)(wrow + (off < last_off ? off : last_off));
     }
   };
-  // The first read of W is issued before x is staged: the two latencies overlap.
-  load_w(0, a_cur);
+  // The first chunk of x and the whole ring are requested together.  The order
+  // (x, then the ring's places in turn) is the one every pass of the loop below
+  // leaves behind, so the compiler's count of reads in flight is exact there.
   stage_load(0);
-  stage_store(0);
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) {
+    load_w(d * 128, ring[d]);
+    asm volatile("" ::: "memory");
+  }
+  stage_store(0, 0);
   __syncthreads();
 
-  for (int c = 0; c < chunks; ++c) {
+  int c = 0;
+  do {  // a slice has at least one chunk; a loop that may run zero times lets the first reads sink below the barrier
     const int buf = c & 1;
-    if (c + 1 < chunks) stage_load(c + 1);  // in flight while this chunk is multiplied
+    stage_load(c + 1);  // in flight while this chunk is multiplied
+    asm volatile("" ::: "memory");  // issued before the ring's reads, so that waiting for it leaves those in flight
 #pragma unroll
-    for (int it = 0; it < SK_KC / 128; ++it) {
-      const int koff = c * SK_KC + it * 128;
-      load_w(koff + 128, a_nxt);  // past the slice's end this reads nothing (zeros)
+    for (int d = 0; d < DEPTH; ++d) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int col = it * 128 + j * 32 + kb * 8;
+        const int col = d * 128 + j * 32 + kb * 8;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           SkFrag b;
           b.u4 = *(const uint4*)(&xs[buf][mt * 16 + r16][col]);
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[j].v, b.v, acc[mt], 0, 0, 0);
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[d][j].v, b.v, acc[mt], 0, 0, 0);
         }
       }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) a_cur[j] = a_nxt[j];
+      load_w((c + 1) * SK_KC + d * 128, ring[d]);  // the same place of the ring, one chunk on
+      asm volatile("" ::: "memory");               // here, and not gathered at the chunk's end
     }
-    if (c + 1 < chunks) {
-      stage_store(buf ^ 1);  // the other buffer was last read in chunk c - 1, before the barrier below
-      __syncthreads();
-    }
-  }
+    stage_store(c + 1, buf ^ 1);  // that buffer was last read in chunk c - 1, before the barrier below
+    __syncthreads();
+  } while (++c < chunks);
 
   if (!wave_has_rows) return;
   // a lane holds the sums for x row m = mt*16 + r16 and W rows n0 + kb*4 .. + 3
@@ -183,9 +217,23 @@ __global__ void sk_reduce_kernel(const float* __restrict__ part, TC* __restrict_
 // fills the CUs evenly (close below a multiple of their number), with about
 // 2048 waves in all and slices that are not too short.
 #define SK_NUM_CUS 256
+// For measurements: a plan that replaces the model's for every shape (0, 0 = the model's again).
+static int sk_forced_waves = 0, sk_forced_units = 0;
+extern "C" void rv_gemm_skinny_force_plan(int waves, int units_per_slice) {
+  sk_forced_waves = waves >= 4 && waves <= SK_MAX_WAVES ? waves : 0;
+  sk_forced_units = units_per_slice > 0 ? units_per_slice : 0;
+}
+
 extern "C" void rv_gemm_skinny_plan(int N, int K, int* waves, int* slices, int* slice_len) {
   const int tiles = rv_div_up(N, 16);
   const int units = rv_div_up(K, 128);
+  if (sk_forced_waves && sk_forced_units) {
+    const int per = sk_forced_units < units ? sk_forced_units : units;
+    *waves = sk_forced_waves;
+    *slice_len = per * 128;
+    *slices = rv_div_up(units, per);
+    return;
+  }
   double best_time = 1e300;
   int best_w = 4, best_len = units * 128, best_s = 1;
   const double w_bytes = 2.0 * N * K;
