@@ -42,11 +42,18 @@ __device__ __forceinline__ float rv_to_float(bf16_t x) {
   return __uint_as_float(((uint32_t)x.bits) << 16);
 }
 
+// Round to nearest even, NaN stays NaN: gfx950 has an instruction for it
+// (v_cvt_pk_bf16_f32), which the cast compiles to.
 __device__ __forceinline__ uint16_t rv_f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // NaN stays NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+
+// Two values in one register, `lo` in the low half: one instruction.
+__device__ __forceinline__ uint32_t rv_pack_bf16x2(float lo, float hi) {
+  typedef float rv_float2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 rv_bf16x2_t __attribute__((ext_vector_type(2)));
+  const rv_float2_t f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, rv_bf16x2_t));
 }
 
 template <typename T>
