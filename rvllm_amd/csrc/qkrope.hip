@@ -14,56 +14,150 @@
 //             page = table[req, pos / page_size], in the layout of kv_layout.h
 //             (the reference writes at the same point: fused_rope_partial_f16kv.cu:69-91);
 //             a negative page skips the write
-// Norm, angle, sine and cosine are 32-bit.
+// Norm, angle, sine and cosine are 32-bit.  The sines and cosines of a step's
+// tokens are the same in every layer that rotates alike, so they come from a
+// table made once a step (rope_table_kernel) instead of being worked out
+// again in every layer.
 #include "common.h"
 #include "kv_layout.h"
 
 #define QKR_MAX_HD 512
+#define QKR_PAIRS (QKR_MAX_HD / 2 / RV_WAVE)  // pairs (i, i + hd/2) a lane holds at most
 
-// One value of the projection's output: stored as T, or the sum of `slices`
-// 32-bit partial sums (the K slices of the product), added in their order.
+// cos_out[t][i] = cos(float(positions[t]) * inv_freq[i]), sin alike; i < half.
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, const int* __restrict__ positions,
+                                  float* __restrict__ cos_out, float* __restrict__ sin_out, int num_tokens, int half) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)num_tokens * half) return;
+  const int t = (int)(idx / half);
+  const int i = (int)(idx - (long long)t * half);
+  const float angle = (float)positions[t] * inv_freq[i];
+  float s, c;
+  sincosf(angle, &s, &c);
+  cos_out[idx] = c;
+  sin_out[idx] = s;
+}
+
+extern "C" int rv_rope_table(hipStream_t stream, const float* inv_freq, const int* positions, float* cos_out,
+                             float* sin_out, int num_tokens, int half) {
+  RV_CHECK(num_tokens >= 0 && half > 0 && inv_freq && positions && cos_out && sin_out, "rope_table: bad arguments");
+  if (num_tokens == 0) return 0;
+  const long long total = (long long)num_tokens * half;
+  rope_table_kernel<<<dim3((unsigned)rv_div_up(total, 256)), dim3(256), 0, stream>>>(inv_freq, positions, cos_out,
+                                                                                     sin_out, num_tokens, half);
+  RV_LAUNCH_CHECK("rope_table");
+  return 0;
+}
+
+// Values src[d] of one head for d = i and i + half, i = lane + 64 j: stored as
+// T, or the sums of `slices` 32-bit partial sums (the K slices of the
+// product), added in their order, four reads of a place in flight at a time.
 template <typename T>
-__device__ __forceinline__ float qkr_input(const void* qkv, int slices, long long slice_stride, size_t at) {
-  if (slices == 0) return rv_to_float(((const T*)qkv)[at]);
-  const float* p = (const float*)qkv + at;
-  float sum = 0.f;
-  int s = 0;
-  for (; s + 4 <= slices; s += 4) {  // four loads in flight, added in the order of the slices
-    const float a = p[(size_t)s * slice_stride], b = p[(size_t)(s + 1) * slice_stride];
-    const float c = p[(size_t)(s + 2) * slice_stride], d = p[(size_t)(s + 3) * slice_stride];
-    sum = (((sum + a) + b) + c) + d;
+__device__ __forceinline__ void qkr_load(const void* qkv, int slices, long long slice_stride, size_t src, int lane,
+                                         int half, float (&lo)[QKR_PAIRS], float (&hi)[QKR_PAIRS]) {
+#pragma unroll
+  for (int j = 0; j < QKR_PAIRS; ++j) lo[j] = hi[j] = 0.f;
+  if (slices == 0) {
+    const T* p = (const T*)qkv + src;
+#pragma unroll
+    for (int j = 0; j < QKR_PAIRS; ++j) {
+      const int i = lane + j * RV_WAVE;
+      if (i < half) {
+        lo[j] = rv_to_float(p[i]);
+        hi[j] = rv_to_float(p[i + half]);
+      }
+    }
+    return;
   }
-  for (; s < slices; ++s) sum += p[(size_t)s * slice_stride];
-  return sum;
+  const float* p = (const float*)qkv + src;
+  int s = 0;
+  for (; s + 4 <= slices; s += 4) {
+    float a[4][QKR_PAIRS], b[4][QKR_PAIRS];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float* ps = p + (size_t)(s + u) * slice_stride;
+#pragma unroll
+      for (int j = 0; j < QKR_PAIRS; ++j) {
+        const int i = lane + j * RV_WAVE;
+        const int at = i < half ? i : 0;  // a lane past the end reads a valid place and drops it
+        a[u][j] = ps[at];
+        b[u][j] = ps[at + half];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+#pragma unroll
+      for (int j = 0; j < QKR_PAIRS; ++j) {
+        lo[j] += a[u][j];
+        hi[j] += b[u][j];
+      }
+    }
+  }
+  for (; s < slices; ++s) {
+    const float* ps = p + (size_t)s * slice_stride;
+#pragma unroll
+    for (int j = 0; j < QKR_PAIRS; ++j) {
+      const int i = lane + j * RV_WAVE;
+      const int at = i < half ? i : 0;
+      lo[j] += ps[at];
+      hi[j] += ps[at + half];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < QKR_PAIRS; ++j)
+    if (lane + j * RV_WAVE >= half) lo[j] = hi[j] = 0.f;
 }
 
 template <typename T>
 __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int slices, long long slice_stride,
                                              T* __restrict__ q_out,
                                              const void* __restrict__ q_w, const void* __restrict__ k_w, int w_f32,
-                                             float eps, float offset, const float* __restrict__ inv_freq, int rot,
+                                             float eps, float offset, const float* __restrict__ rope_cos,
+                                             const float* __restrict__ rope_sin, int rot,
                                              const int* __restrict__ positions, const int* __restrict__ token_req,
                                              const int* __restrict__ block_table, int table_width,
                                              T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size,
                                              int num_pages, int nq, int nkv, int hd, int write_kv) {
-  __shared__ float buf[4][QKR_MAX_HD];
   const int wave = threadIdx.x / RV_WAVE;
   const int lane = threadIdx.x & (RV_WAVE - 1);
   const int t = blockIdx.x;
   const int head = blockIdx.y * 4 + wave;
   const int total_heads = nq + 2 * nkv;
-  if (head >= total_heads) return;  // whole wave leaves together; no block barrier below
+  if (head >= total_heads) return;  // whole wave leaves together; there is no block barrier below
 
   const size_t src = (size_t)t * total_heads * hd + (size_t)head * hd;  // first element of this head in qkv
   const bool is_q = head < nq;
   const bool is_k = !is_q && head < nq + nkv;
-  const int pos = positions[t];
+  const int half = hd / 2;
+  const int rot_half = rot / 2;
+
+  // The head's values, the angles' cosines and sines and the norm's weights are
+  // asked for before anything waits (on the position, the table, the page).
+  float lo[QKR_PAIRS], hi[QKR_PAIRS];
+  qkr_load<T>(qkv, slices, slice_stride, src, lane, half, lo, hi);
+  float c[QKR_PAIRS], s[QKR_PAIRS], w_lo[QKR_PAIRS], w_hi[QKR_PAIRS];
+  const void* w = is_q ? q_w : k_w;
+  const bool rotates = rot_half > 0 && (is_q || is_k);
+#pragma unroll
+  for (int j = 0; j < QKR_PAIRS; ++j) {
+    const int i = lane + j * RV_WAVE;
+    c[j] = 1.f, s[j] = 0.f, w_lo[j] = 0.f, w_hi[j] = 0.f;
+    if (rotates && i < rot_half) {
+      c[j] = rope_cos[(size_t)t * rot_half + i];
+      s[j] = rope_sin[(size_t)t * rot_half + i];
+    }
+    if (w != nullptr && !(!is_q && !is_k) && i < half) {
+      w_lo[j] = rv_load_w(w, w_f32, i);
+      w_hi[j] = rv_load_w(w, w_f32, i + half);
+    }
+  }
 
   T* dst = nullptr;
   if (is_q) {
     dst = q_out + ((size_t)t * nq + head) * hd;
   } else {
     if (!write_kv) return;
+    const int pos = positions[t];
     const int req = token_req[t];
     const int logical = pos / page_size;
     if (logical >= table_width) return;
@@ -75,45 +169,42 @@ __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int s
     } else {
       // values are stored as projected, transposed inside the page
       T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
-      for (int d = lane; d < hd; d += RV_WAVE)
-        col[(size_t)d * page_size] = rv_from_float<T>(qkr_input<T>(qkv, slices, slice_stride, src + d));
+#pragma unroll
+      for (int j = 0; j < QKR_PAIRS; ++j) {
+        const int i = lane + j * RV_WAVE;
+        if (i < half) {
+          col[(size_t)i * page_size] = rv_from_float<T>(lo[j]);
+          col[(size_t)(i + half) * page_size] = rv_from_float<T>(hi[j]);
+        }
+      }
       return;
     }
   }
 
-  float* x = buf[wave];
-  const void* w = is_q ? q_w : k_w;
-  float ss = 0.f;
-  for (int d = lane; d < hd; d += RV_WAVE) {
-    const float v = qkr_input<T>(qkv, slices, slice_stride, src + d);
-    x[d] = v;
-    ss += v * v;
-  }
   if (w != nullptr) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < QKR_PAIRS; ++j) ss += lo[j] * lo[j] + hi[j] * hi[j];
     ss = rv_wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
-    for (int d = lane; d < hd; d += RV_WAVE) {
-      x[d] = x[d] * inv * (offset + rv_load_w(w, w_f32, d));
+#pragma unroll
+    for (int j = 0; j < QKR_PAIRS; ++j) {
+      lo[j] = lo[j] * inv * (offset + w_lo[j]);
+      hi[j] = hi[j] * inv * (offset + w_hi[j]);
     }
   }
-  __builtin_amdgcn_wave_barrier();
-  __threadfence_block();
-
-  const int half = hd / 2;
-  const int rot_half = rot / 2;
-  for (int i = lane; i < half; i += RV_WAVE) {
-    const float a = x[i];
-    const float b = x[i + half];
+#pragma unroll
+  for (int j = 0; j < QKR_PAIRS; ++j) {
+    const int i = lane + j * RV_WAVE;
+    if (i >= half) continue;
+    float a = lo[j], b = hi[j];
     if (i < rot_half) {
-      const float angle = (float)pos * inv_freq[i];
-      float s, c;
-      sincosf(angle, &s, &c);
-      dst[i] = rv_from_float<T>(a * c - b * s);
-      dst[i + half] = rv_from_float<T>(a * s + b * c);
-    } else {
-      dst[i] = rv_from_float<T>(a);
-      dst[i + half] = rv_from_float<T>(b);
+      const float ra = a * c[j] - b * s[j];
+      const float rb = a * s[j] + b * c[j];
+      a = ra, b = rb;
     }
+    dst[i] = rv_from_float<T>(a);
+    dst[i + half] = rv_from_float<T>(b);
   }
 }
 
@@ -121,8 +212,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int s
 // partial sums [slices][tokens][...], slice_stride elements apart.
 extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int slices, long long slice_stride,
                                         void* q_out, const void* q_w,
-                                        const void* k_w, int w_f32, float eps, float offset, const float* inv_freq,
-                                        int rot, const int* positions, const int* token_req, const int* block_table,
+                                        const void* k_w, int w_f32, float eps, float offset, const float* rope_cos,
+                                        const float* rope_sin, int rot, const int* positions, const int* token_req, const int* block_table,
                                         int table_width, void* k_pages, void* v_pages, int page_size, int num_pages,
                                         int dtype, int num_tokens, int nq, int nkv, int hd, int write_kv) {
   RV_CHECK(num_tokens >= 0 && nq > 0 && nkv > 0, "qk_norm_rope: bad sizes T=%d nq=%d nkv=%d", num_tokens, nq, nkv);
@@ -131,7 +222,7 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
   RV_CHECK(hd >= 2 && hd % 2 == 0 && hd <= QKR_MAX_HD, "qk_norm_rope: head_dim %d must be even and <= %d", hd,
            QKR_MAX_HD);
   RV_CHECK(rot >= 0 && rot <= hd && rot % 2 == 0, "qk_norm_rope: rotary_dim %d must be even and <= head_dim %d", rot, hd);
-  RV_CHECK(rot == 0 || inv_freq != nullptr, "qk_norm_rope: rotation needs inverse frequencies");
+  RV_CHECK(rot == 0 || (rope_cos != nullptr && rope_sin != nullptr), "qk_norm_rope: rotation needs the table of cosines and sines");
   RV_CHECK((q_w == nullptr) == (k_w == nullptr), "qk_norm_rope: query and key norm weights come together");
   RV_CHECK(!write_kv || (page_size > 0 && num_pages > 0 && table_width > 0 && block_table && k_pages && v_pages),
            "qk_norm_rope: cache write needs pages and a block table");
@@ -139,11 +230,11 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
   dim3 grid(num_tokens, rv_div_up(nq + 2 * nkv, 4)), block(4 * RV_WAVE);
   if (dtype == RV_F32)
     qk_norm_rope_kv_write_kernel<float><<<grid, block, 0, stream>>>(
-        qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, inv_freq, rot, positions, token_req,
+        qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions, token_req,
         block_table, table_width, (float*)k_pages, (float*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv);
   else if (dtype == RV_BF16)
     qk_norm_rope_kv_write_kernel<bf16_t><<<grid, block, 0, stream>>>(
-        qkv, slices, slice_stride, (bf16_t*)q_out, q_w, k_w, w_f32, eps, offset, inv_freq, rot, positions, token_req,
+        qkv, slices, slice_stride, (bf16_t*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions, token_req,
         block_table, table_width, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv);
   else
     return rv_fail("qk_norm_rope: unsupported dtype %d", dtype);

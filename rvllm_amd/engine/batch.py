@@ -52,6 +52,8 @@ class StepBatch:
     num_logit_rows: int = 0
     host_q_start: Optional[np.ndarray] = None
     host_chunk_start: Optional[np.ndarray] = None
+    # what parts work out once a step and share between layers (keyed by who made it)
+    shared: dict = dataclasses.field(default_factory=dict)
 
     @property
     def decode_only(self) -> bool:

@@ -93,7 +93,7 @@ class ModelRunner:
             # The first step of a shape runs eagerly and is then recorded
             # (recording runs nothing) for the steps that follow.
             logits = self.model.forward(batch, self.storage.views)
-            shaped = dataclasses.replace(batch, max_context=key[1])
+            shaped = dataclasses.replace(batch, max_context=key[1], shared={})  # nothing made outside the recording
             graph = torch.cuda.CUDAGraph()
             torch.cuda.synchronize()
             with torch.cuda.graph(graph, pool=self._graph_pool):

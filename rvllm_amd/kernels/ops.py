@@ -241,14 +241,30 @@ def gemm_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Ten
     return out
 
 
+def rope_table(inv_freq: torch.Tensor, positions: torch.Tensor, num_tokens: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """(cos, sin) of float(position) * inv_freq[i] for the first ``num_tokens``
+    positions: two 32-bit tensors ``[num_tokens, len(inv_freq)]``."""
+    _gpu(inv_freq, positions)
+    _i32(positions)
+    _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and inv_freq.numel() > 0, "rope_table: bad inv_freq")
+    _need(positions.numel() >= num_tokens, "rope_table: positions too short")
+    half = inv_freq.numel()
+    cos = torch.empty((num_tokens, half), dtype=torch.float32, device=inv_freq.device)
+    sin = torch.empty_like(cos)
+    _check(library().rv_rope_table(_stream(), _ptr(inv_freq), _ptr(positions), _ptr(cos), _ptr(sin), _c_int(num_tokens),
+                                   _c_int(half)))
+    return cos, sin
+
+
 def qk_norm_rope_kv_write(qkv, q_out: torch.Tensor, q_weight: Optional[torch.Tensor],
                           k_weight: Optional[torch.Tensor], eps: float, offset: float,
-                          inv_freq: Optional[torch.Tensor], rotary_dim: int, positions: torch.Tensor,
+                          rope: Optional[tuple[torch.Tensor, torch.Tensor]], rotary_dim: int, positions: torch.Tensor,
                           token_req: torch.Tensor, block_table: Optional[torch.Tensor],
                           k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], num_q_heads: int,
                           num_kv_heads: int, head_dim: int, write_kv: bool = True) -> torch.Tensor:
     qptr, slices, stride, n, qkv_width, qkv_dtype = _branch_args(qkv, "qk_norm_rope")
-    _gpu(q_out, q_weight, k_weight, inv_freq, positions, token_req, block_table, k_pages, v_pages)
+    rope_cos, rope_sin = rope if rope is not None else (None, None)
+    _gpu(q_out, q_weight, k_weight, rope_cos, rope_sin, positions, token_req, block_table, k_pages, v_pages)
     _i32(positions, token_req)
     _need(qkv_width == (num_q_heads + 2 * num_kv_heads) * head_dim, "qk_norm_rope: bad qkv shape")
     _need(q_out.shape == (n, num_q_heads * head_dim) and q_out.dtype == qkv_dtype, "qk_norm_rope: bad q_out")
@@ -259,8 +275,10 @@ def qk_norm_rope_kv_write(qkv, q_out: torch.Tensor, q_weight: Optional[torch.Ten
               "qk_norm_rope: bad norm weights")
         _need(q_weight.dtype == k_weight.dtype, "qk_norm_rope: norm weights must share a dtype")
         w_f32 = int(q_weight.dtype == torch.float32)
-    if inv_freq is not None:
-        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() >= rotary_dim // 2, "qk_norm_rope: bad inv_freq")
+    if rope is not None:
+        for table in (rope_cos, rope_sin):
+            _need(table.dtype == torch.float32 and table.is_contiguous() and table.shape == (n, rotary_dim // 2),
+                  f"qk_norm_rope: the table of cosines and sines must be 32-bit [{n}, {rotary_dim // 2}]")
     page_size = num_pages = width = 0
     if write_kv:
         _need(k_pages is not None and v_pages is not None and block_table is not None, "qk_norm_rope: no cache given")
@@ -272,7 +290,7 @@ def qk_norm_rope_kv_write(qkv, q_out: torch.Tensor, q_weight: Optional[torch.Ten
     _check(library().rv_qk_norm_rope_kv_write(
         _stream(), qptr, _c_int(slices), _c_ll(stride), _ptr(q_out), _ptr(q_weight), _ptr(k_weight), _c_int(w_f32),
         _c_float(eps),
-        _c_float(offset), _ptr(inv_freq), _c_int(rotary_dim if inv_freq is not None else 0), _ptr(positions),
+        _c_float(offset), _ptr(rope_cos), _ptr(rope_sin), _c_int(rotary_dim if rope is not None else 0), _ptr(positions),
         _ptr(token_req), _ptr(block_table), _c_int(width), _ptr(k_pages), _ptr(v_pages), _c_int(page_size),
         _c_int(num_pages), _dt(q_out), _c_int(n), _c_int(num_q_heads), _c_int(num_kv_heads), _c_int(head_dim),
         _c_int(int(write_kv))))

@@ -82,7 +82,7 @@ class PagedAttention(Mixer):
         norm = self.qk_norm or {}
         ops.qk_norm_rope_kv_write(
             qkv, q, self.q_norm_w, self.k_norm_w, float(norm.get("eps", 0.0)),
-            1.0 if norm.get("unit_offset", False) else 0.0, self.position.inv_freq(x.device),
+            1.0 if norm.get("unit_offset", False) else 0.0, self.position.tables(step),
             self.position.rotary_dim, step.positions, step.token_req, table, cache.k_pages, cache.v_pages,
             self.num_heads, self.num_kv_heads, self.head_dim, write_kv=cache.writes)
         attn = torch.empty_like(q)

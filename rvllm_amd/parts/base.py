@@ -135,13 +135,18 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """How a mixer marks positions.  ``kernel_args`` gives what the fused
-    query/key kernel needs: the number of rotated dimensions and the table of
-    inverse frequencies (already divided by any scaling factor)."""
+    """How a mixer marks positions.  ``rotary_dim`` is the number of rotated
+    dimensions of a head and ``tables(step)`` the 32-bit cosines and sines of
+    the step's tokens, ``([tokens, rotary_dim / 2], the same)``, or None when
+    nothing is rotated: what the fused query/key kernel needs.  Layers that
+    rotate alike share one pair of tables per step (``step.shared``)."""
 
     rotary_dim: int = 0
 
     def inv_freq(self, device: torch.device) -> Optional[torch.Tensor]:
+        return None
+
+    def tables(self, step: "StepBatch") -> Optional[tuple[torch.Tensor, torch.Tensor]]:
         return None
 
 

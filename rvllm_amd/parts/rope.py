@@ -6,7 +6,8 @@ uses the head size, not the number of rotated dimensions
 Dividing the inverse frequencies by ``factor`` is the linear scaling of the
 global layers: the angle of position p becomes that of p / factor.  The table
 is computed in 64-bit and rounded to 32-bit once; the angle
-``float(pos) * inv_freq[i]`` and its sine and cosine are 32-bit in the kernel.
+``float(pos) * inv_freq[i]`` and its sine and cosine are 32-bit in the kernel
+that tabulates them for a step's tokens.
 """
 
 from __future__ import annotations
@@ -41,6 +42,23 @@ class RotaryEncoding(PositionEncoding):
         if self._table is None or self._table.device != torch.device(device):
             self._table = self.inv_freq_host().to(device)
         return self._table
+
+
+    def tables(self, step):
+        """Cosines and sines of this step's tokens, made once a step for all
+        the layers with these parameters."""
+        if self.rotary_dim == 0:
+            return None
+        shared = getattr(step, "shared", None)
+        key = ("rope", self.theta, self.factor, self.rotary_dim, self.head_dim)
+        if shared is not None and key in shared:
+            return shared[key]
+        from ..kernels import ops
+
+        made = ops.rope_table(self.inv_freq(step.positions.device), step.positions, step.num_tokens)
+        if shared is not None:
+            shared[key] = made
+        return made
 
 
 class NoPositionEncoding(PositionEncoding):

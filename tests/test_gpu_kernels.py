@@ -201,7 +201,8 @@ def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size):
     inv_freq = (10000.0 ** (-2.0 * torch.arange(rot // 2, dtype=torch.float64) / hd) / 4.0).float()
     q_out = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
     kp_dev, vp_dev = to_cache(k_pages, v_pages)
-    ops.qk_norm_rope_kv_write(dev(qkv), q_out, dev(qw), dev(kw), 1e-6, 1.0, dev(inv_freq) if rot else None, rot,
+    rope = ops.rope_table(dev(inv_freq), dev(positions), T) if rot else None
+    ops.qk_norm_rope_kv_write(dev(qkv), q_out, dev(qw), dev(kw), 1e-6, 1.0, rope, rot,
                               dev(positions), dev(torch.zeros(T, dtype=torch.int32)), dev(table), kp_dev, vp_dev, nq,
                               nkv, hd)
     kp, vp = from_cache(kp_dev, vp_dev)
@@ -224,6 +225,18 @@ def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size):
     for page, off in written:
         mask[page, off] = False
     assert kp.cpu()[mask].abs().sum() == 0 and vp.cpu()[mask].abs().sum() == 0
+
+
+def test_rope_table_against_64_bit_angles():
+    """cos and sin of float32(position) * inv_freq, positions up to a long context, against 64-bit
+    functions of the same 32-bit angle."""
+    inv_freq = (1e6 ** (-2.0 * torch.arange(24, dtype=torch.float64) / 48) / 8.0).float()
+    positions = torch.tensor([0, 1, 2, 17, 1023, 4096, 65535, 131071, 5, 99999], dtype=torch.int32)
+    cos, sin = ops.rope_table(dev(inv_freq), dev(positions), 8)  # fewer tokens than positions: only the first 8
+    assert cos.shape == sin.shape == (8, 24) and cos.dtype == torch.float32
+    angle = (positions[:8].float()[:, None] * inv_freq[None, :]).double()  # the product is rounded to 32-bit first
+    assert torch.allclose(cos.cpu().double(), angle.cos(), atol=2e-7, rtol=0)
+    assert torch.allclose(sin.cpu().double(), angle.sin(), atol=2e-7, rtol=0)
 
 
 def test_qk_norm_rope_without_cache_write_leaves_the_cache_alone():

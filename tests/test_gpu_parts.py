@@ -49,8 +49,18 @@ def test_rope_part_tables():
     rope = POSITION_ENCODINGS.build(PartSpec("rope", {"theta": 5e5, "factor": 4.0}), head_dim=32)
     assert rope.rotary_dim == 32
     assert torch.equal(rope.inv_freq(DEV).cpu(), P.rope_inv_freq(32, 5e5, 4.0))
+    # the step's tables: made once and shared by parts with the same parameters, not by others
+    import types
+    step = types.SimpleNamespace(positions=torch.tensor([3, 4, 900], dtype=torch.int32, device=DEV), num_tokens=3,
+                                 shared={})
+    cos, sin = rope.tables(step)
+    angle = torch.tensor([3.0, 4.0, 900.0])[:, None] * P.rope_inv_freq(32, 5e5, 4.0)[None, :]
+    assert torch.allclose(cos.cpu(), angle.cos(), atol=1e-6) and torch.allclose(sin.cpu(), angle.sin(), atol=1e-6)
+    twin = POSITION_ENCODINGS.build(PartSpec("rope", {"theta": 5e5, "factor": 4.0}), head_dim=32)
+    other = POSITION_ENCODINGS.build(PartSpec("rope", {"theta": 5e5, "factor": 1.0}), head_dim=32)
+    assert twin.tables(step)[0] is cos and other.tables(step)[0] is not cos and len(step.shared) == 2
     none = POSITION_ENCODINGS.build(PartSpec("none"), head_dim=32)
-    assert none.rotary_dim == 0 and none.inv_freq(DEV) is None
+    assert none.rotary_dim == 0 and none.inv_freq(DEV) is None and none.tables(step) is None
     with pytest.raises(ValueError):
         POSITION_ENCODINGS.build(PartSpec("rope", {"theta": 1e4, "rotary_dim": 7}), head_dim=32)
 
