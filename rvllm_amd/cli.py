@@ -29,7 +29,7 @@ ENV_WHITELIST = {
     "RVLLM_MODEL_DIR", "RVLLM_GEN_PROMPT_FILE", "RVLLM_GEN_PROMPT", "RVLLM_GEN_TOKENS", "RVLLM_GEN_DUMP",
     "RVLLM_SAMPLE_T", "RVLLM_SAMPLE_TOPK", "RVLLM_SAMPLE_TOPP", "RVLLM_SAMPLE_SEED", "RVLLM_EOS",
     "RVLLM_DEFAULT_MAX_TOKENS", "RVLLM_DRY_RUN", "RVLLM_MAX_INFLIGHT_REQUESTS", "RVLLM_DTYPE",
-    "RVLLM_AMD_BUILD_DIR",
+    "RVLLM_AMD_BUILD_DIR", "RVLLM_GRAPHS",
 }
 
 USAGE = """usage: rvllm-amd --model DIR [options]
@@ -51,6 +51,7 @@ USAGE = """usage: rvllm-amd --model DIR [options]
   --ignore-eos                   keep going past an end id
   --dump FILE                    write the generated ids, one request per line         [$RVLLM_GEN_DUMP]
   --random-weights CONFIG.json   no folder: random weights for this configuration (with --weights-seed S)
+  --graphs                       replay decode steps from captured HIP graphs (bfloat16)  [$RVLLM_GRAPHS]
   --dry-run                      check the configuration and the arguments, load nothing
 """
 
@@ -88,6 +89,7 @@ def parse(argv: list[str], env: dict) -> dict:
         "eos": env.get("RVLLM_EOS", ""), "ignore_eos": False, "dump": env.get("RVLLM_GEN_DUMP"),
         "random_weights": None, "weights_seed": 0,
         "dry_run": env.get("RVLLM_DRY_RUN", "") not in ("", "0", "false"),
+        "graphs": env.get("RVLLM_GRAPHS", "") not in ("", "0", "false"),
     }
     ints = {"--max-model-len", "--max-num-seqs", "--max-inflight-requests", "--max-num-batched-tokens",
             "--max-prefill-chunk", "--page-size", "--max-cache-tokens", "--prompt-len", "--max-tokens", "--top-k",
@@ -102,7 +104,7 @@ def parse(argv: list[str], env: dict) -> dict:
             raise UsageError(USAGE)
         if key in ("--host", "--port", "--backend", "--served-model-name", "--system-prompt", "--system-prompt-file"):
             raise UsageError(f"{key}: this build has no HTTP server; prompts come from --prompt-file or --prompt-ids")
-        if key in ("--dry-run", "--ignore-eos"):
+        if key in ("--dry-run", "--ignore-eos", "--graphs"):
             o[key[2:].replace("-", "_")] = True
             continue
         if key not in ints | floats | strings | {"--prompt-ids"}:
@@ -171,7 +173,8 @@ def main(argv=None, env=None) -> int:
 
         cfg = EngineConfig(dtype=o["dtype"], page_size=o["page_size"], max_model_len=o["max_model_len"],
                            max_num_seqs=o["max_num_seqs"], max_num_batched_tokens=o["max_num_batched_tokens"],
-                           max_prefill_chunk=o["max_prefill_chunk"], max_cache_tokens=o["max_cache_tokens"]).validate()
+                           max_prefill_chunk=o["max_prefill_chunk"], max_cache_tokens=o["max_cache_tokens"],
+                           use_graphs=o["graphs"]).validate()
         if o["random_weights"]:
             doc = json.loads(Path(o["random_weights"]).read_text())
             arch = architecture_of(doc, o["random_weights"])

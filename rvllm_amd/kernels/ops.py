@@ -9,6 +9,7 @@ back to a library: if the kernel library cannot be loaded the call raises.
 from __future__ import annotations
 
 import ctypes
+import functools
 import threading
 from typing import Optional
 
@@ -330,9 +331,16 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
 
 MFMA_ATTENTION_MAX_HEAD_DIM = 256
 MFMA_ATTENTION_MAX_GROUP = 16
-# Units (waves) a launch aims for: the kernel runs one wave a SIMD, 1024 at once on 256 CUs; a few more
-# even out units of different length.
-_ATTENTION_TARGET_UNITS = 1536
+# What the split plan of the decode kernel knows about the machine (measured on MI355X with keys and values of
+# 256 per head; microseconds): the kernel runs one wave a SIMD, 1024 at once on 256 CUs; a wave takes about 3.2
+# for a block of 32 keys when it waits for nobody; 1024 waves together stream about 6.3 TB/s; launches, the first
+# reads and the merge cost about 10.6 (7 without a merge), and the merge 0.1 more per split.
+_ATTN_WAVE_SLOTS = 1024
+_ATTN_BLOCK_US = 3.2
+_ATTN_BYTES_PER_US = 6.3e6
+_ATTN_FIXED_US = 10.6
+_ATTN_FIXED_UNSPLIT_US = 7.0
+_ATTN_MERGE_US_PER_SPLIT = 0.1
 
 
 def mfma_attention_covers(k_pages: torch.Tensor, v_pages: torch.Tensor, num_q_heads: int) -> bool:
@@ -341,11 +349,19 @@ def mfma_attention_covers(k_pages: torch.Tensor, v_pages: torch.Tensor, num_q_he
             and num_q_heads % nkv == 0 and num_q_heads // nkv <= MFMA_ATTENTION_MAX_GROUP)
 
 
+@functools.lru_cache(maxsize=4096)
 def plan_attention_splits(num_requests: int, max_portion: int, max_context: int, nkv: int, group: int,
-                          window: Optional[int]) -> tuple[int, int, int]:
+                          window: Optional[int], head_dim: int = 256) -> tuple[int, int, int]:
     """(tiles per request, number of key splits, keys per split) for the
-    matrix-core kernel.  A tile is 16 / group_pad tokens of one request and one
-    key/value head; its keys are split so that about 2048 waves run."""
+    matrix-core decode kernel.  A tile is 16 / group_pad tokens of one request
+    and one key/value head; its keys are split over waves.
+
+    The number of splits is the one a small model of the machine likes best:
+    the waves run in rounds of 1024 (one a SIMD); a round takes what its
+    longest wave takes alone or what its bytes take at full streaming rate,
+    whichever is longer; a last round that is not full still takes a wave's
+    whole time, which is why 1.3 rounds are worse than 1 or 2; every split
+    adds to the merge."""
     group_pad = 1
     while group_pad < group:
         group_pad *= 2
@@ -355,11 +371,26 @@ def plan_attention_splits(num_requests: int, max_portion: int, max_context: int,
     if window:
         # first key of a tile rounded down to 32, up to the tile's last token
         span = min(span, window - 1 + 31 + tokens_per_tile)
-    span = -(-span // 32) * 32
+    blocks = -(-span // 32)
     units = num_requests * tiles * nkv
-    splits = 1 if units >= 512 else min(-(-_ATTENTION_TARGET_UNITS // units), span // 32)
-    split_len = -(-(-(-span // splits)) // 32) * 32
-    return tiles, -(-span // split_len), split_len
+    block_bytes = 32 * head_dim * 2 * 2  # keys and values of a block, bf16
+    best = None
+    for splits in range(1, min(blocks, 512) + 1):
+        per = -(-blocks // splits)  # blocks a split
+        if per * (splits - 1) >= blocks:
+            continue  # the last split would be empty: the same plan as with fewer splits
+        waves = units * splits
+        full_rounds, rest = divmod(waves, _ATTN_WAVE_SLOTS)
+        alone = per * _ATTN_BLOCK_US
+        time = full_rounds * max(alone, _ATTN_WAVE_SLOTS * per * block_bytes / _ATTN_BYTES_PER_US)
+        if rest:  # fewer waves draw less than the full rate: about its square root of their share
+            rate = _ATTN_BYTES_PER_US * (rest / _ATTN_WAVE_SLOTS) ** 0.5
+            time += max(alone, rest * per * block_bytes / rate)
+        time += _ATTN_FIXED_US + _ATTN_MERGE_US_PER_SPLIT * splits if splits > 1 else _ATTN_FIXED_UNSPLIT_US
+        if best is None or time < best[0] * (1.0 - 1e-9):
+            best = (time, splits, per * 32)
+    _, splits, split_len = best
+    return tiles, splits, split_len
 
 
 # Portions of at least this many tokens go to the kernel whose blocks share key
@@ -420,7 +451,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                      _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_int(portion_min), _c_float(scale)))
     if shortest_rest > 0:
         tiles, num_splits, split_len = plan_attention_splits(step.num_requests, shortest_rest, step.max_context, nkv,
-                                                             group, window)
+                                                             group, window, hd)
         if splits is not None:
             num_splits, split_len = splits
             need = -(-step.max_context // 32) * 32
