@@ -75,6 +75,33 @@ __device__ __forceinline__ float rv_round_to(float x) {
   return rv_to_float(rv_from_float<T>(x));
 }
 
+// Gated activations, act(gate) * up; ACT 0: gelu in its tanh form
+// (v3/kernels/fused_gelu_mul_f16.cu:20-27), ACT 1: silu.  The 32-bit path uses
+// the accurate library functions.  Where the result is rounded to bf16 anyway,
+// tanh(y) = 1 - 2 / (1 + e^2y) with the hardware's exponential and reciprocal
+// (an error of some 1e-6) costs a fifth of that; every bf16 kernel that
+// applies an activation goes through here, so they all round alike.
+template <typename T, int ACT>
+__device__ __forceinline__ float rv_gated(float gate, float up);
+template <>
+__device__ __forceinline__ float rv_gated<float, 0>(float z, float up) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))) * up;
+}
+template <>
+__device__ __forceinline__ float rv_gated<float, 1>(float z, float up) {
+  return z / (1.0f + expf(-z)) * up;
+}
+template <>
+__device__ __forceinline__ float rv_gated<bf16_t, 0>(float z, float up) {
+  const float y = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  const float t = 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * y));  // e^2y = inf gives 1, 0 gives -1
+  return 0.5f * z * (1.0f + t) * up;
+}
+template <>
+__device__ __forceinline__ float rv_gated<bf16_t, 1>(float z, float up) {
+  return z * __frcp_rn(1.0f + __expf(-z)) * up;
+}
+
 // A weight vector that may be stored in either type (norm weights keep the
 // type they were stored in).
 __device__ __forceinline__ float rv_load_w(const void* w, int is_f32, int i) {

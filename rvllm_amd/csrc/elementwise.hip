@@ -341,10 +341,6 @@ extern "C" int rv_add_rmsnorm(hipStream_t stream, const void* branch, int slices
 // gated activation: out[t,i] = act(gu[t,i]) * gu[t,I+i]
 // act 0: gelu, tanh form; act 1: silu
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ float rv_gelu_tanh(float z) {
-  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-}
-__device__ __forceinline__ float rv_silu(float z) { return z / (1.0f + expf(-z)); }
 
 template <typename T, int V, int ACT>
 __global__ void gated_act_kernel(const void* __restrict__ gu, int slices, long long slice_stride, T* __restrict__ out,
@@ -359,7 +355,7 @@ __global__ void gated_act_kernel(const void* __restrict__ gu, int slices, long l
   row_load_branch<T, V>(gu, slices, slice_stride, at, g);
   row_load_branch<T, V>(gu, slices, slice_stride, at + inter, u);
 #pragma unroll
-  for (int v = 0; v < V; ++v) g[v] = (ACT == 0 ? rv_gelu_tanh(g[v]) : rv_silu(g[v])) * u[v];
+  for (int v = 0; v < V; ++v) g[v] = rv_gated<T, ACT>(g[v], u[v]);
   row_store<T, V>(out + (size_t)t * inter + i, g);
 }
 

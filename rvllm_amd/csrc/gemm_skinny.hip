@@ -60,7 +60,12 @@ __device__ __forceinline__ void sk_store1<uint16_t>(uint16_t* p, float a) {
 
 // grid (row blocks, K slices); block = waves x 64.  With one slice the result
 // goes to `out` as TC; with more, slice s writes 32-bit sums to part[s][M][N].
-template <int MT, typename TC>
+// ACT < 0: x is [M, K].  ACT 0 or 1: x is [M, 2K], the gates beside the ups as
+// the product before left them, and what is multiplied is act(gate) * up,
+// worked out while a piece of x is staged (rounded to bf16 there, exactly as
+// the separate kernel for it would store it): a kernel and a pass over memory
+// less.  Every block of rows repeats that work, so it pays for few rows only.
+template <int MT, typename TC, int ACT = -1>
 __global__ void __launch_bounds__(SK_MAX_WAVES * 64)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, TC* __restrict__ out,
                    float* __restrict__ part, int M, int N, int K, long long ldx, long long ldw, long long ldc,
@@ -92,6 +97,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   // a thread holds at most PIECES / 256 pieces (blocks have at least 4 waves)
   constexpr int MAX_REGS = (PIECES + 255) / 256;
   uint4 staged[MAX_REGS];
+  uint4 staged_up[ACT >= 0 ? MAX_REGS : 1];
   const int last_k = kend - 8;  // the last 16-byte piece of this slice (slices are multiples of 8 long)
   auto stage_load = [&](int c) {
 #pragma unroll
@@ -103,6 +109,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
       m = m < M ? m : M - 1;
       k = k < last_k ? k : last_k;
       staged[n] = *(const uint4*)(x + (size_t)m * ldx + k);
+      if constexpr (ACT >= 0) staged_up[n] = *(const uint4*)(x + (size_t)m * ldx + K + k);
     }
   };
   auto stage_store = [&](int c, int buf) {
@@ -120,6 +127,19 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
       // The staged values count as used only from here on: otherwise the masking
       // drifts up between the products, and its wait for x drains the ring.
       asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+      if (ACT >= 0 && m < M) {  // rows past M are never stored: no activation for them
+        uint4 u = staged_up[n];
+        asm volatile("" : "+v"(u.x), "+v"(u.y), "+v"(u.z), "+v"(u.w));
+        const uint32_t gw[4] = {v.x, v.y, v.z, v.w}, uw[4] = {u.x, u.y, u.z, u.w};
+        uint32_t r[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float lo = rv_gated<bf16_t, ACT>(__uint_as_float(gw[i] << 16), __uint_as_float(uw[i] << 16));
+          const float hi = rv_gated<bf16_t, ACT>(__uint_as_float(gw[i] & 0xffff0000u), __uint_as_float(uw[i] & 0xffff0000u));
+          r[i] = rv_pack_bf16x2(lo, hi);
+        }
+        v = make_uint4(r[0], r[1], r[2], r[3]);
+      }
       v.x &= keep, v.y &= keep, v.z &= keep, v.w &= keep;
       *(uint4*)(&xs[buf][m][col]) = v;
     }
@@ -279,14 +299,14 @@ extern "C" int rv_gemm_skinny_slices(int N, int K) {
   return slices;
 }
 
-template <int MT, typename TC>
+template <int MT, typename TC, int ACT = -1>
 static int sk_launch(hipStream_t stream, const uint16_t* x, const uint16_t* w, TC* out, float* part, int M, int N,
                      int K, long long ldx, long long ldw, long long ldc, int do_reduce) {
   int waves, slices, len;
   rv_gemm_skinny_plan(N, K, &waves, &slices, &len);
   if (slices > 1 && part == nullptr) return rv_fail("gemm_skinny: this shape needs a workspace");
   dim3 grid(rv_div_up(rv_div_up(N, 16), waves), slices);
-  gemm_skinny_kernel<MT, TC><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc, len);
+  gemm_skinny_kernel<MT, TC, ACT><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc, len);
   RV_LAUNCH_CHECK("gemm_skinny");
   if (slices > 1 && do_reduce) {
     const long long total = (long long)M * N;
@@ -324,6 +344,28 @@ extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, 
   }
 #undef SK_CASE
   return rv_fail("gemm_skinny: unsupported output dtype %d", out_dtype);
+}
+
+// The product of act(gate) * up with W: x is [M, 2K] (gates, then ups), M at most 16.
+// act 0: gelu in its tanh form, 1: silu.  Otherwise as rv_gemm_skinny.
+extern "C" int rv_gemm_skinny_gated(hipStream_t stream, const void* x, const void* w, void* out, int out_dtype,
+                                    float* part, int M, int N, int K, long long ldx, long long ldw, long long ldc,
+                                    int do_reduce, int act) {
+  RV_CHECK(M >= 0 && M <= 16 && N > 0 && K > 0, "gemm_skinny_gated: M=%d must be at most 16 (N=%d K=%d)", M, N, K);
+  RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny_gated: K and the row strides must be multiples of 8");
+  RV_CHECK(ldx >= 2ll * K && ldw >= K && ldc >= N, "gemm_skinny_gated: leading dimensions too small");
+  RV_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny_gated: operands must be 16-byte aligned");
+  RV_CHECK(act == 0 || act == 1, "gemm_skinny_gated: unknown activation %d", act);
+  if (M == 0) return 0;
+  const uint16_t* xp = (const uint16_t*)x;
+  const uint16_t* wp = (const uint16_t*)w;
+  if (out_dtype == RV_F32)
+    return act == 0 ? sk_launch<1, float, 0>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc, do_reduce)
+                    : sk_launch<1, float, 1>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc, do_reduce);
+  if (out_dtype == RV_BF16)
+    return act == 0 ? sk_launch<1, uint16_t, 0>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc, do_reduce)
+                    : sk_launch<1, uint16_t, 1>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc, do_reduce);
+  return rv_fail("gemm_skinny_gated: unsupported output dtype %d", out_dtype);
 }
 
 // out[m][n] (bf16 or 32-bit) = sum over slices of part[s][m][n].

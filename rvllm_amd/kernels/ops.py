@@ -544,3 +544,37 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
 
 
 SKINNY_MAX_ROWS = 64
+GATED_GEMM_MAX_ROWS = 16
+
+
+def gemm_bf16_gated(gate_up: torch.Tensor, w: torch.Tensor, activation: str, out_dtype: Optional[torch.dtype] = None,
+                    sliced_ok: bool = False):
+    """(act(gate) * up) @ w^T for a bf16 ``gate_up`` of ``[rows, 2K]`` (gates, then ups) with few rows: the
+    activation is applied while the product stages its input, which saves a kernel and a pass over memory.  None
+    when this kernel does not cover the case (the caller then applies ``gated_act`` and multiplies)."""
+    if not isinstance(gate_up, torch.Tensor) or gate_up.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return None
+    m, two_k = gate_up.shape
+    n, k = w.shape
+    if m > GATED_GEMM_MAX_ROWS or two_k != 2 * k or k % 8 or gate_up.stride(1) != 1 or w.stride(1) != 1:
+        return None
+    if (m > 1 and gate_up.stride(0) % 8) or (n > 1 and w.stride(0) % 8) or gate_up.data_ptr() % 16 or w.data_ptr() % 16:
+        return None
+    _need(gate_up.is_cuda and w.is_cuda, "gemm: arguments must live on the GPU")
+    _need(activation in ACTIVATIONS, f"gemm_bf16_gated: unknown activation {activation!r}")
+    lib = library()
+    out_dtype = out_dtype or gate_up.dtype
+    ldx = gate_up.stride(0) if m > 1 else two_k
+    ldw = w.stride(0) if n > 1 else k
+    slices = lib.rv_gemm_skinny_slices(_c_int(n), _c_int(k))
+    act = _c_int(ACTIVATIONS[activation])
+    if sliced_ok and slices > 1:
+        part = torch.empty((slices, m, n), dtype=torch.float32, device=w.device)
+        _check(lib.rv_gemm_skinny_gated(_stream(), _ptr(gate_up), _ptr(w), None, _c_int(_DT[out_dtype]), _ptr(part),
+                                        _c_int(m), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(n), _c_int(0), act))
+        return SlicedSums(part, out_dtype)
+    out = torch.empty((m, n), dtype=out_dtype, device=w.device)
+    part = torch.empty(slices * m * n, dtype=torch.float32, device=w.device) if slices > 1 else None
+    _check(lib.rv_gemm_skinny_gated(_stream(), _ptr(gate_up), _ptr(w), _ptr(out), _dt(out), _ptr(part), _c_int(m),
+                                    _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(n), _c_int(1), act))
+    return out

@@ -16,6 +16,9 @@ from .registry import FEED_FORWARDS
 from .spec import PartSpec
 
 
+FUSED_ACTIVATION_MAX_ROWS = 4
+
+
 class GatedMLP(FeedForward):
     def __init__(self, spec: PartSpec, *, hidden_size: int):
         self.hidden_size = int(hidden_size)
@@ -42,6 +45,12 @@ class GatedMLP(FeedForward):
 
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
         gate_up = linear(x, self.w_gate_up, sliced_ok=True)
+        # a few rows in bf16: the down product applies the activation itself while it stages its input
+        # (measured on MI355X: a gain up to 4 rows, a loss from 8 on, where every block repeats too much of it)
+        if x.shape[0] <= FUSED_ACTIVATION_MAX_ROWS:
+            fused = ops.gemm_bf16_gated(gate_up, self.w_down, self.activation, sliced_ok=True)
+            if fused is not None:
+                return fused
         act = ops.gated_act(gate_up, self.activation)
         return linear(act, self.w_down, sliced_ok=True)
 

@@ -152,6 +152,32 @@ def test_gemm_skinny(m, n, k, out_dtype):
     assert torch.equal(one[0], out[m - 1])
 
 
+@pytest.mark.parametrize("activation", ["gelu_pytorch_tanh", "silu"])
+@pytest.mark.parametrize("m,n,k", [(1, 40, 64), (8, 96, 1416), (16, 2560, 10240), (5, 33, 520)])
+def test_gemm_with_the_gated_activation_in_its_staging(m, n, k, activation):
+    """(act(gate) * up) @ W^T in one kernel: against 64-bit arithmetic, and bit for bit against the
+    activation kernel followed by the product (both round the activation to bf16 the same way)."""
+    g = torch.Generator().manual_seed(22)
+    gate_up = (torch.randn(m, 2 * k, generator=g) * 1.5).bfloat16()
+    gate_up[0, :4] = torch.tensor([-30.0, 30.0, 0.0, -0.0]).bfloat16()  # the ends of the activation's range
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    fused = ops.gemm_bf16_gated(dev(gate_up), dev(w), activation, out_dtype=torch.float32)
+    assert fused is not None and fused.shape == (m, n)
+    gd, ud = gate_up[:, :k].double(), gate_up[:, k:].double()
+    act = F.gelu(gd, approximate="tanh") if activation != "silu" else F.silu(gd)
+    want = (act * ud).bfloat16().double() @ w.double().T
+    scale = want.abs().max().item()
+    assert (fused.cpu().double() - want).abs().max().item() <= 2e-3 * scale * max(1.0, math.sqrt(k) / 16)
+    two_step = ops.gemm_bf16(ops.gated_act(dev(gate_up), activation), dev(w), out_dtype=torch.float32)
+    assert torch.equal(fused, two_step)
+    # unreduced slices, as the norm after it takes them
+    sums = ops.gemm_bf16_gated(dev(gate_up), dev(w), activation, sliced_ok=True)
+    assert torch.allclose(ops.as_tensor(sums).float(), fused, atol=2e-2 * scale, rtol=0)
+    # more rows than it covers, or another type: left to the two kernels
+    assert ops.gemm_bf16_gated(dev(torch.zeros(17, 2 * k).bfloat16()), dev(w), activation) is None
+    assert ops.gemm_bf16_gated(dev(gate_up.float()), dev(w.float()), activation) is None
+
+
 def test_gemm_skinny_reads_strided_rows_and_refuses_what_it_cannot():
     g = torch.Generator().manual_seed(21)
     big = dev(torch.randn(6, 96, generator=g).bfloat16())
