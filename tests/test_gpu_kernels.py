@@ -402,6 +402,60 @@ def test_paged_attention_shared_tiles_long_prompt_portions():
         assert torch.allclose(case.run("mfma", 1.0 / 16).float(), want, **tol(torch.bfloat16)), (portions, window)
 
 
+def _plant(case, b, key, head, dim, value):
+    """Key `key` of request b becomes `value` at one dimension and nothing else, in the log and in the pages."""
+    k = case.k_all[b]
+    k[key, head] = 0
+    k[key, head, dim] = value
+    case.k_log[int(case.table[b, key // case.page_size]), key % case.page_size, head] = k[key, head]
+
+
+@pytest.mark.parametrize("far", [0, 17, 31, 32, 63, 64, 200, 255])
+def test_shared_tiles_attention_finds_one_key(far):
+    """The kernel for prompt portions: one key carries all the weight for every later token, wherever it
+    lies in a 64-key stage (first or second half, which different waves multiply and then merge) and
+    whichever stage; tokens before it do not see it; at a window's edge it is seen, one further not."""
+    nq, nkv, hd, n = 4, 2, 64, 256
+    for window in (None, 40):
+        case = Case([(0, n)], nq, nkv, hd, 16, torch.bfloat16, 14, window, drop_passed_pages=False)
+        for b in range(1):
+            case.k_all[b] *= 0.01
+            case.k_log *= 0.01
+        _plant(case, 0, far, 1, 5, 40.0)
+        case.q[:] = 0
+        case.q[:, :, 5] = 40.0  # every query looks along dimension 5
+        got = case.run("mfma", 1.0, prefill_kernel=True).float()
+        want = case.reference(1.0).float()
+        assert torch.allclose(got, want, **tol(torch.bfloat16))
+        v_far = case.v_all[0][far, 1].float()
+        for t in (far, min(far + 39, n - 1), min(far + 40, n - 1), n - 1):
+            sees = t >= far and (window is None or t - far < window)
+            hit = torch.allclose(got[t, 2:], v_far.expand(2, hd), atol=2e-2)  # heads 2, 3 read kv head 1
+            assert hit == sees, (far, window, t)
+
+
+def test_shared_tiles_attention_when_the_maximum_grows_late():
+    """Scores that grow along the sequence by more than the step at which sums are rescaled, by less than
+    it, and not at all: the running sums follow in each case."""
+    nq, nkv, hd, n = 2, 1, 32, 320
+    for step_size in (0.0, 0.05, 3.0, 9.0):
+        case = Case([(0, n)], nq, nkv, hd, 16, torch.bfloat16, 15, None)
+        ramp = torch.arange(n, dtype=torch.float32) / 32 * step_size  # grows by step_size per 32 keys
+        case.k_all[0][:, 0, 7] = ramp.to(torch.bfloat16)
+        for j in range(n):
+            case.k_log[int(case.table[0, j // 16]), j % 16, 0, 7] = case.k_all[0][j, 0, 7]
+        case.q[:, :, 7] = 1.0
+        got = case.run("mfma", 1.0, prefill_kernel=True).float()
+        assert torch.allclose(got, case.reference(1.0).float(), **tol(torch.bfloat16)), step_size
+
+
+def test_shared_tiles_attention_missing_page_shows():
+    case = Case([(0, 100)], 2, 1, 32, 16, torch.bfloat16, 16)
+    case.table[0, 2] = -1  # keys 32..47 are gone: every token from 32 on must not look valid
+    got = case.run("mfma", 1.0, prefill_kernel=True)
+    assert torch.isnan(got[32:]).all() and not torch.isnan(got[:32]).any()
+
+
 @pytest.mark.parametrize("splits", [(1, 224), (2, 128), (7, 32), (4, 64)])
 @pytest.mark.parametrize("window", [None, 100])
 def test_paged_attention_mfma_every_split(splits, window):
