@@ -251,7 +251,7 @@ def main() -> int:
     }
     if not args.no_prefill:
         T = args.prefill_tokens
-        psec = time_prefill(parts, T, repeats=2)
+        psec = time_prefill(parts, T, repeats=5)
         flops = T * layer_flops_per_token + attention_flops(cfg, 0, T) + head_flops_per_row
         result["prefill"] = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
                              "frac": round(flops / psec / PEAK_FLOPS[short], 4)}

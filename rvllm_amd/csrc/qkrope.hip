@@ -208,6 +208,142 @@ __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int s
   }
 }
 
+// The same work for head sizes that are multiples of 8 up to 256 (and rotated
+// widths that are multiples of 8): a lane holds 4 neighbouring dimensions, so
+// it reads and writes 8 or 16 bytes at a time instead of 2 or 4, and gets the
+// other half of its pairs from the lane hd/8 away.
+template <typename T>
+struct QkrVec;
+template <>
+struct QkrVec<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 x = *(const float4*)p;
+    v[0] = x.x, v[1] = x.y, v[2] = x.z, v[3] = x.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <>
+struct QkrVec<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+    const uint2 x = *(const uint2*)p;
+    v[0] = __uint_as_float(x.x << 16), v[1] = __uint_as_float(x.x & 0xffff0000u);
+    v[2] = __uint_as_float(x.y << 16), v[3] = __uint_as_float(x.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+    *(uint2*)p = make_uint2(rv_pack_bf16x2(v[0], v[1]), rv_pack_bf16x2(v[2], v[3]));
+  }
+};
+
+template <typename T>
+__global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, int slices, long long slice_stride,
+                                                 T* __restrict__ q_out, const void* __restrict__ q_w,
+                                                 const void* __restrict__ k_w, int w_f32, float eps, float offset,
+                                                 const float* __restrict__ rope_cos, const float* __restrict__ rope_sin,
+                                                 int rot, const int* __restrict__ positions,
+                                                 const int* __restrict__ token_req, const int* __restrict__ block_table,
+                                                 int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                                 int page_size, int num_pages, int nq, int nkv, int hd, int write_kv) {
+  const int wave = threadIdx.x / RV_WAVE;
+  const int lane = threadIdx.x & (RV_WAVE - 1);
+  const int t = blockIdx.x;
+  const int head = blockIdx.y * 4 + wave;
+  const int total_heads = nq + 2 * nkv;
+  if (head >= total_heads) return;  // whole wave leaves together; there is no block barrier below
+
+  const size_t src = (size_t)t * total_heads * hd + (size_t)head * hd;  // first element of this head in qkv
+  const bool is_q = head < nq;
+  const bool is_k = !is_q && head < nq + nkv;
+  const int half_lanes = hd / 8;          // lanes that hold one half of the head
+  const bool active = lane < 2 * half_lanes;
+  const int d0 = active ? lane * 4 : 0;   // a lane without dimensions reads a valid place and drops it
+  const bool first_half = lane < half_lanes;
+  const int i0 = first_half ? d0 : d0 - hd / 2;  // index of the lane's pairs
+  const int rot_half = rot / 2;
+
+  // the head's values: stored as T, or the sums of the product's K slices in their order
+  float x[4] = {0.f, 0.f, 0.f, 0.f};
+  if (slices == 0) {
+    QkrVec<T>::load((const T*)qkv + src + d0, x);
+  } else {
+    const float* p = (const float*)qkv + src + d0;
+    int s = 0;
+    for (; s + 4 <= slices; s += 4) {  // four reads in flight
+      const float4 a = *(const float4*)(p + (size_t)s * slice_stride);
+      const float4 b = *(const float4*)(p + (size_t)(s + 1) * slice_stride);
+      const float4 c = *(const float4*)(p + (size_t)(s + 2) * slice_stride);
+      const float4 d = *(const float4*)(p + (size_t)(s + 3) * slice_stride);
+      x[0] = (((x[0] + a.x) + b.x) + c.x) + d.x;
+      x[1] = (((x[1] + a.y) + b.y) + c.y) + d.y;
+      x[2] = (((x[2] + a.z) + b.z) + c.z) + d.z;
+      x[3] = (((x[3] + a.w) + b.w) + c.w) + d.w;
+    }
+    for (; s < slices; ++s) {
+      const float4 a = *(const float4*)(p + (size_t)s * slice_stride);
+      x[0] += a.x, x[1] += a.y, x[2] += a.z, x[3] += a.w;
+    }
+  }
+  if (!active) x[0] = x[1] = x[2] = x[3] = 0.f;
+
+  const void* w = is_q ? q_w : k_w;
+  const bool normed = w != nullptr && (is_q || is_k);
+  const bool rotates = (is_q || is_k) && active && i0 < rot_half;
+  float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f}, g[4] = {0.f, 0.f, 0.f, 0.f};
+  if (rotates) {
+    QkrVec<float>::load(rope_cos + (size_t)t * rot_half + i0, c);
+    QkrVec<float>::load(rope_sin + (size_t)t * rot_half + i0, sn);
+  }
+  if (normed) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) g[j] = rv_load_w(w, w_f32, d0 + j);
+  }
+
+  T* dst = nullptr;
+  if (is_q) {
+    dst = q_out + ((size_t)t * nq + head) * hd;
+  } else {
+    if (!write_kv) return;
+    const int pos = positions[t];
+    const int req = token_req[t];
+    const int logical = pos / page_size;
+    if (logical >= table_width) return;
+    const int page = block_table[(size_t)req * table_width + logical];
+    if (page < 0 || page >= num_pages) return;
+    const int slot = pos % page_size;
+    if (is_k) {
+      dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
+    } else {
+      // values are stored as projected, transposed inside the page
+      T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
+      if (active) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) col[(size_t)(d0 + j) * page_size] = rv_from_float<T>(x[j]);
+      }
+      return;
+    }
+  }
+
+  if (normed) {
+    float ss = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+    ss = rv_wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) x[j] = x[j] * inv * (offset + g[j]);
+  }
+  if (rot_half > 0) {
+    // the other half of each pair sits hd/8 lanes away; every lane takes part in the exchange
+    const int partner = first_half ? lane + half_lanes : lane - half_lanes;
+    const int from = active ? partner : lane;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float other = __shfl(x[j], from, RV_WAVE);
+      if (rotates) x[j] = first_half ? x[j] * c[j] - other * sn[j] : x[j] * c[j] + other * sn[j];
+    }
+  }
+  if (active) QkrVec<T>::store(dst + d0, x);
+}
+
 // `slices` 0: qkv holds T values [tokens, (nq + 2 nkv) * hd]; otherwise 32-bit
 // partial sums [slices][tokens][...], slice_stride elements apart.
 extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int slices, long long slice_stride,
@@ -228,6 +364,22 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
            "qk_norm_rope: cache write needs pages and a block table");
   if (num_tokens == 0) return 0;
   dim3 grid(num_tokens, rv_div_up(nq + 2 * nkv, 4)), block(4 * RV_WAVE);
+  if (hd % 8 == 0 && hd <= 4 * RV_WAVE && rot % 8 == 0) {  // four dimensions a lane
+    if (dtype == RV_F32)
+      qk_norm_rope_kv_write_vec_kernel<float><<<grid, block, 0, stream>>>(
+          qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions,
+          token_req, block_table, table_width, (float*)k_pages, (float*)v_pages, page_size, num_pages, nq, nkv, hd,
+          write_kv);
+    else if (dtype == RV_BF16)
+      qk_norm_rope_kv_write_vec_kernel<bf16_t><<<grid, block, 0, stream>>>(
+          qkv, slices, slice_stride, (bf16_t*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions,
+          token_req, block_table, table_width, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, num_pages, nq, nkv, hd,
+          write_kv);
+    else
+      return rv_fail("qk_norm_rope: unsupported dtype %d", dtype);
+    RV_LAUNCH_CHECK("qk_norm_rope_kv_write");
+    return 0;
+  }
   if (dtype == RV_F32)
     qk_norm_rope_kv_write_kernel<float><<<grid, block, 0, stream>>>(
         qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions, token_req,

@@ -215,7 +215,8 @@ def from_cache(kp, vp):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nq,nkv,hd,rot", [(4, 2, 16, 16), (6, 3, 48, 48), (5, 1, 80, 40), (8, 4, 256, 256), (3, 3, 128, 0)])
+@pytest.mark.parametrize("nq,nkv,hd,rot", [(4, 2, 16, 16), (6, 3, 48, 48), (5, 1, 80, 40), (8, 4, 256, 256), (3, 3, 128, 0),
+                                          (2, 1, 36, 12), (2, 2, 512, 512)])  # the last two: the kernel for odd sizes
 @pytest.mark.parametrize("page_size", [16, 64])
 def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size):
     T = 37
