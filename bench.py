@@ -2,6 +2,7 @@
 """Decode and prefill throughput of the engine at Gemma-3-4B layer sizes.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
+    python bench.py --workload 12b|27b [--requests N] [--layers L]     (another measurement, see WORKLOADS)
 
 Default run: the layer sizes of the 4B-sized configuration (34 layers, 5
 sliding : 1 global, hidden 2560, 8 query / 4 key-value heads of 256, GeGLU
@@ -158,6 +159,60 @@ def time_prefill(engine_parts, length: int, repeats: int):
     return best
 
 
+# The engine workloads of the larger configurations: requests through the scheduler, prompts cut into portions
+# and mixed with decoding.  (requests, prompt lengths from .. to, new tokens, portion)
+WORKLOADS = {
+    "12b": (dict(num_hidden_layers=48, hidden_size=3840, num_attention_heads=16, num_key_value_heads=8, head_dim=256,
+                 intermediate_size=15360, query_pre_attn_scalar=256), 64, (512, 4096), 256, 2048),
+    "27b": (dict(num_hidden_layers=62, hidden_size=5376, num_attention_heads=32, num_key_value_heads=16, head_dim=128,
+                 intermediate_size=21504, query_pre_attn_scalar=168), 32, (16384, 16384), 128, 2048),
+}
+
+
+def run_workload(name: str, requests, layers) -> int:
+    """Generates through the whole engine (scheduler, portions, decoding) and prints one JSON line."""
+    import torch
+
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.config.gemma3 import Gemma3Config
+    from rvllm_amd.engine.engine import LLMEngine
+    from rvllm_amd.sampling.params import SamplingParams
+    import rvllm_amd.models  # noqa: F401
+
+    sizes, n_req, (lo, hi), new, portion = WORKLOADS[name]
+    n_req = requests or n_req
+    doc = dict(GEMMA3_4B, **sizes)
+    full_layers = doc["num_hidden_layers"]
+    if layers:
+        doc["num_hidden_layers"] = layers
+    cfg = Gemma3Config.from_dict(doc, "workload configuration")
+    g = torch.Generator().manual_seed(3)
+    lengths = [int(torch.randint(lo, hi + 1, (1,), generator=g)) for _ in range(n_req)]
+    prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lengths]
+    engine_cfg = EngineConfig(dtype="bfloat16", page_size=16, max_model_len=max(lengths) + new + 16, max_num_seqs=n_req,
+                              max_num_batched_tokens=portion + n_req, max_prefill_chunk=portion,
+                              max_cache_tokens=sum(lengths) + n_req * (new + 32), use_graphs=True)
+    log(f"building the {name}-sized model ({cfg.num_hidden_layers} layers) with random weights")
+    engine = LLMEngine.from_random(cfg, 0, engine_cfg)
+    engine.runner.warm_up([portion])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    results = engine.generate(prompts, [SamplingParams() for _ in prompts], new, (), True)
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    made = sum(len(r.tokens) for r in results)
+    print(json.dumps({
+        "metric": f"tokens/s through the engine, {name}-sized workload", "value": round((sum(lengths) + made) / sec, 1),
+        "unit": "tok/s", "n_gpus": 1, "seconds": round(sec, 2), "higher_is_better": True, "dtype": "bf16",
+        "data": "synthetic: random weights, uniform token ids, greedy",
+        "config": {"model": f"gemma3-{name}-sized dense decoder", "requests": n_req, "prompt_tokens": sum(lengths),
+                   "new_tokens": made, "portion": portion, "layers": cfg.num_hidden_layers,
+                   "layers_of_named_config": full_layers, "hidden_size": cfg.hidden_size, "head_dim": cfg.head_dim,
+                   "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads},
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -171,10 +226,15 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--graphs", type=int, default=1, help="replay decode steps from captured HIP graphs (0 = off)")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), help="instead of the default run: an engine workload of a "
+                    "larger configuration (requests through the scheduler); --requests and --layers shrink it")
+    ap.add_argument("--requests", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
+    if args.workload:
+        return run_workload(args.workload, args.requests, args.layers if args.layers != FULL_LAYERS else 0)
 
     import torch
 
