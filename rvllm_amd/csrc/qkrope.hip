@@ -167,6 +167,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int s
     if (is_k) {
       dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
     } else {
+      if (write_kv == 2) return;  // values are written a page at a time by v_write_pages_kernel
       // values are stored as projected, transposed inside the page
       T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
 #pragma unroll
@@ -314,6 +315,7 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
     if (is_k) {
       dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
     } else {
+      if (write_kv == 2) return;  // values are written a page at a time by v_write_pages_kernel
       // values are stored as projected, transposed inside the page
       T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
       if (active) {
@@ -344,6 +346,73 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
   if (active) QkrVec<T>::store(dst + d0, x);
 }
 
+// The values of a step's tokens, written a page at a time.  Values lie
+// transposed inside a page (kv_layout.h), so the kernels above, a wave per
+// token and head, scatter them two or four bytes at a time; for prompt
+// portions that is most of their time.  Here a block takes one page of one
+// request and one key/value head: thread d gathers the page's tokens at
+// dimension d (for a fixed token the threads read one contiguous row) and writes
+// row d of the page, 16 bytes at a time when the portion covers the whole page.
+// grid (pages a portion may touch, kv heads, requests).
+template <typename T>
+__global__ void __launch_bounds__(256)
+v_write_pages_kernel(const T* __restrict__ qkv, T* __restrict__ v_pages, const int* __restrict__ q_start,
+                     const int* __restrict__ chunk_start, const int* __restrict__ block_table, int table_width,
+                     int page_size, int num_pages, int nq, int nkv, int hd) {
+  const int b = blockIdx.z, kvh = blockIdx.y;
+  const int q0 = q_start[b];
+  const int n = q_start[b + 1] - q0;
+  const int s = chunk_start[b];
+  if (n <= 0) return;
+  const int lp = s / page_size + blockIdx.x;
+  const int lo = s > lp * page_size ? s : lp * page_size;
+  const int hi = s + n < (lp + 1) * page_size ? s + n : (lp + 1) * page_size;
+  if (lo >= hi || lp >= table_width) return;
+  const int page = block_table[(size_t)b * table_width + lp];
+  if (page < 0 || page >= num_pages) return;
+  const size_t width = (size_t)(nq + 2 * nkv) * hd;
+  const T* src = qkv + (size_t)(q0 + lo - s) * width + (size_t)(nq + nkv + kvh) * hd;  // token at position lo
+  const int slot0 = lo - lp * page_size;
+  constexpr int VEC = 16 / sizeof(T);  // elements of a 16-byte store
+  const bool whole = hi - lo == page_size && page_size % VEC == 0;
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    T* row = v_pages + rv_v_index(page, kvh, 0, d, nkv, page_size, hd);
+    if (whole) {
+      for (int g = 0; g < page_size; g += VEC) {
+        T v[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = src[(size_t)(g + i) * width + d];
+        *(uint4*)(row + g) = *(const uint4*)v;
+      }
+    } else {
+      for (int i = 0; i < hi - lo; ++i) row[slot0 + i] = src[(size_t)i * width + d];
+    }
+  }
+}
+
+extern "C" int rv_v_write_pages(hipStream_t stream, const void* qkv, void* v_pages, const int* q_start,
+                                const int* chunk_start, const int* block_table, int table_width, int page_size,
+                                int num_pages, int dtype, int num_requests, int max_portion, int nq, int nkv, int hd) {
+  RV_CHECK(num_requests >= 0 && max_portion >= 1 && nq > 0 && nkv > 0 && hd > 0, "v_write_pages: bad sizes");
+  RV_CHECK(page_size > 0 && num_pages > 0 && table_width > 0 && qkv && v_pages && q_start && chunk_start && block_table,
+           "v_write_pages: needs the projection's output, the pages and the step's tables");
+  RV_CHECK(num_requests <= 65535 && nkv <= 65535, "v_write_pages: too many requests or heads for one launch");
+  if (num_requests == 0) return 0;
+  // a portion of n tokens touches at most (n - 1) / page_size + 2 pages
+  dim3 grid((max_portion - 1) / page_size + 2, nkv, num_requests);
+  if (dtype == RV_F32)
+    v_write_pages_kernel<float><<<grid, dim3(256), 0, stream>>>((const float*)qkv, (float*)v_pages, q_start, chunk_start,
+                                                               block_table, table_width, page_size, num_pages, nq, nkv, hd);
+  else if (dtype == RV_BF16)
+    v_write_pages_kernel<bf16_t><<<grid, dim3(256), 0, stream>>>((const bf16_t*)qkv, (bf16_t*)v_pages, q_start,
+                                                                chunk_start, block_table, table_width, page_size,
+                                                                num_pages, nq, nkv, hd);
+  else
+    return rv_fail("v_write_pages: unsupported dtype %d", dtype);
+  RV_LAUNCH_CHECK("v_write_pages");
+  return 0;
+}
+
 // `slices` 0: qkv holds T values [tokens, (nq + 2 nkv) * hd]; otherwise 32-bit
 // partial sums [slices][tokens][...], slice_stride elements apart.
 extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int slices, long long slice_stride,
@@ -363,7 +432,9 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
   RV_CHECK(!write_kv || (page_size > 0 && num_pages > 0 && table_width > 0 && block_table && k_pages && v_pages),
            "qk_norm_rope: cache write needs pages and a block table");
   if (num_tokens == 0) return 0;
-  dim3 grid(num_tokens, rv_div_up(nq + 2 * nkv, 4)), block(4 * RV_WAVE);
+  // write_kv 0: nothing goes to the cache; 1: keys and values; 2: keys only (values by rv_v_write_pages)
+  RV_CHECK(write_kv >= 0 && write_kv <= 2, "qk_norm_rope: write_kv is 0, 1 or 2");
+  dim3 grid(num_tokens, rv_div_up(write_kv == 1 ? nq + 2 * nkv : nq + nkv, 4)), block(4 * RV_WAVE);
   if (hd % 8 == 0 && hd <= 4 * RV_WAVE && rot % 8 == 0) {  // four dimensions a lane
     if (dtype == RV_F32)
       qk_norm_rope_kv_write_vec_kernel<float><<<grid, block, 0, stream>>>(

@@ -254,6 +254,40 @@ def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size):
     assert kp.cpu()[mask].abs().sum() == 0 and vp.cpu()[mask].abs().sum() == 0
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [16, 32])
+def test_values_written_a_page_at_a_time(dtype, page_size):
+    """Portions that begin and end inside pages, cover whole pages, and single tokens: the values reach the same
+    places as when every token writes its own, and nothing else is touched."""
+    nq, nkv, hd = 4, 2, 48
+    portions = [(5, 70), (64, 32), (0, 1), (31, 2), (100, 16)]  # (first position, tokens)
+    case = Case(portions, nq, nkv, hd, page_size, dtype, 17)
+    T = case.q.shape[0]
+    g = torch.Generator().manual_seed(18)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd, generator=g).to(dtype)
+    results = []
+    for by_page in (False, True):
+        kp, vp = to_cache(torch.zeros_like(case.k_log), torch.zeros_like(case.v_log))
+        q_out = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
+        ops.qk_norm_rope_kv_write(dev(qkv), q_out, None, None, 0.0, 0.0, None, 0, case.step.positions,
+                                  case.step.token_req, dev(case.table), kp, vp, nq, nkv, hd, values_by_page=by_page)
+        if by_page:
+            assert vp.abs().sum() == 0  # the keys-only mode leaves the values alone
+            ops.v_write_pages(dev(qkv), vp, dev(case.table), case.step, nq, nkv, hd)
+        results.append((q_out.cpu(), kp.cpu(), vp.cpu()))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    # and the values are the projection's, at the token's page and slot
+    _, vp = from_cache(results[1][1].to(DEV), results[1][2].to(DEV))
+    t = 0
+    for b, (s, n) in enumerate(portions):
+        for pos in range(s, s + n):
+            page = int(case.table[b, pos // page_size])
+            want = qkv[t, (nq + nkv) * hd:].view(nkv, hd)
+            assert torch.equal(vp[page, pos % page_size].cpu(), want), (b, pos)
+            t += 1
+
+
 def test_rope_table_against_64_bit_angles():
     """cos and sin of float32(position) * inv_freq, positions up to a long context, against 64-bit
     functions of the same 32-bit angle."""
