@@ -42,9 +42,6 @@ union SkFrag {
 // stride is then 4 banks off a multiple of 64 banks, and the 16 lanes that
 // read the same columns of 16 rows hit 64 different banks.
 #define SK_DEPTH_OF(MT) ((MT) <= 2 ? 4 : 2)
-// Waits until at most n of this wave's reads from memory are still in flight.
-// Reads come back in the order they were issued, so "all but the newest n".
-#define RV_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(0x3F70 | ((n) & 15) | ((((n) >> 4) & 3) << 14))
 #define SK_MAX_WAVES 8
 
 template <typename TC>
