@@ -51,7 +51,7 @@ USAGE = """usage: rvllm-amd --model DIR [options]
   --ignore-eos                   keep going past an end id
   --dump FILE                    write the generated ids, one request per line         [$RVLLM_GEN_DUMP]
   --random-weights CONFIG.json   no folder: random weights for this configuration (with --weights-seed S)
-  --graphs                       replay decode steps from captured HIP graphs (bfloat16)  [$RVLLM_GRAPHS]
+  --no-graphs                    do not replay decode steps from captured HIP graphs   [$RVLLM_GRAPHS=0]
   --dry-run                      check the configuration and the arguments, load nothing
 """
 
@@ -89,7 +89,7 @@ def parse(argv: list[str], env: dict) -> dict:
         "eos": env.get("RVLLM_EOS", ""), "ignore_eos": False, "dump": env.get("RVLLM_GEN_DUMP"),
         "random_weights": None, "weights_seed": 0,
         "dry_run": env.get("RVLLM_DRY_RUN", "") not in ("", "0", "false"),
-        "graphs": env.get("RVLLM_GRAPHS", "") not in ("", "0", "false"),
+        "graphs": env.get("RVLLM_GRAPHS", "1") not in ("0", "false"),
     }
     ints = {"--max-model-len", "--max-num-seqs", "--max-inflight-requests", "--max-num-batched-tokens",
             "--max-prefill-chunk", "--page-size", "--max-cache-tokens", "--prompt-len", "--max-tokens", "--top-k",
@@ -106,6 +106,9 @@ def parse(argv: list[str], env: dict) -> dict:
             raise UsageError(f"{key}: this build has no HTTP server; prompts come from --prompt-file or --prompt-ids")
         if key in ("--dry-run", "--ignore-eos", "--graphs"):
             o[key[2:].replace("-", "_")] = True
+            continue
+        if key == "--no-graphs":
+            o["graphs"] = False
             continue
         if key not in ints | floats | strings | {"--prompt-ids"}:
             raise UsageError(f"unknown argument: {key}")

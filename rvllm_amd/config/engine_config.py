@@ -37,7 +37,7 @@ class EngineConfig:
     # Tokens the cache pool is made for; None = max_num_seqs * max_model_len.
     max_cache_tokens: Optional[int] = None
     # Replay decode-only steps from captured HIP graphs (bf16 only).
-    use_graphs: bool = False
+    use_graphs: bool = True
 
     @property
     def torch_dtype(self) -> torch.dtype:
