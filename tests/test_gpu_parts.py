@@ -17,8 +17,9 @@ from rvllm_amd.engine.batch import BatchBuilder, Portion
 from rvllm_amd.engine.runner import ModelRunner
 from rvllm_amd.kernels import ops
 from rvllm_amd.models import Architecture, register_architecture, unregister_architecture
-from rvllm_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, LayerSpec, Mixer, ModelSpec,
-                             ParamSpec, PartSpec, ScheduleEntry, StateNeed)
+from rvllm_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, FeedForward, LayerSpec, Mixer,
+                             ModelSpec, ParamSpec, PartSpec, PositionEncoding, ScheduleEntry, StateNeed)
+from rvllm_amd.parts.linear import linear
 from rvllm_amd.weights.random_init import random_tensors, write_random_model
 
 pytestmark = pytest.mark.gpu
@@ -306,3 +307,132 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, toy_arch
     runner.release("a2")
     runner.release("b2")
     runner.cache.check()
+
+
+# --------------------------------------------------------------------------
+# A toy feed-forward with routing and a toy position encoding, defined here and
+# plugged in through the registries: no file of the framework changes.
+# --------------------------------------------------------------------------
+class TopOneExperts(FeedForward):
+    """A router picks one of E small gated MLPs per token (router logits in 32-bit)."""
+
+    def __init__(self, spec, *, hidden_size):
+        self.hidden, self.experts, self.inter = hidden_size, int(spec["experts"]), int(spec["intermediate_size"])
+
+    def param_specs(self, prefix):
+        p = f"{prefix}.moe"
+        specs = [ParamSpec(f"{p}.router.weight", (self.experts, self.hidden), init=("normal", 0.5))]
+        for e in range(self.experts):
+            specs += [ParamSpec(f"{p}.experts.{e}.gate_up.weight", (2 * self.inter, self.hidden), init=("normal", 0.2)),
+                      ParamSpec(f"{p}.experts.{e}.down.weight", (self.hidden, self.inter), init=("normal", 0.2))]
+        return specs
+
+    def bind(self, tensors, prefix, device, dtype):
+        p = f"{prefix}.moe"
+        self.router = tensors[f"{p}.router.weight"].to(device=device, dtype=torch.float32)
+        self.gate_up = [tensors[f"{p}.experts.{e}.gate_up.weight"].to(device=device, dtype=dtype) for e in range(self.experts)]
+        self.down = [tensors[f"{p}.experts.{e}.down.weight"].to(device=device, dtype=dtype) for e in range(self.experts)]
+
+    def forward(self, x, step):
+        choice = (x.float() @ self.router.T).argmax(dim=-1)
+        out = torch.zeros_like(x)
+        for e in range(self.experts):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                act = ops.gated_act(linear(x[rows].contiguous(), self.gate_up[e]), "silu")  # the framework's kernels
+                out[rows] = linear(act, self.down[e])
+        return out
+
+
+class RootPositions(PositionEncoding):
+    """Rotation by the angle sqrt(position) * inv_freq[i]: another rule for the angles, the same kernel."""
+
+    def __init__(self, spec, *, head_dim):
+        self.rotary_dim = head_dim
+        self.inv = 50.0 ** (-2.0 * torch.arange(head_dim // 2, dtype=torch.float64) / head_dim)
+
+    def tables(self, step):
+        key = ("root", self.rotary_dim)
+        if key not in step.shared:
+            angle = step.positions[: step.num_tokens].double().sqrt()[:, None] * self.inv.to(step.positions.device)[None, :]
+            step.shared[key] = (angle.cos().float().contiguous(), angle.sin().float().contiguous())
+        return step.shared[key]
+
+
+def toy2_spec(cfg: ToyConfig, prefix="model") -> ModelSpec:
+    norm = PartSpec("rmsnorm", {"eps": 1e-6, "unit_offset": True})
+    attn = PartSpec("attention", {"num_heads": 2, "num_kv_heads": 2, "head_dim": 16, "scale": 0.25, "window": 6,
+                                  "qk_norm": None, "position": PartSpec("root_positions")})
+    dense = PartSpec("gated_mlp", {"intermediate_size": 2 * cfg.hidden, "activation": "silu"})
+    routed = PartSpec("top_one_experts", {"experts": 3, "intermediate_size": cfg.hidden})
+    layers = tuple(LayerSpec(f"{prefix}.layers.{l}", PartSpec("sandwich"), attn, routed if l % 2 else dense, norm)
+                   for l in range(cfg.layers))  # different feed-forwards in different layers
+    return ModelSpec(cfg.architecture, cfg.hidden, cfg.vocab, 512, PartSpec("scaled_embedding", {"scale": 1.0}),
+                     layers, tuple(ScheduleEntry(l) for l in range(cfg.layers)), norm, PartSpec("lm_head", {"tied": True}),
+                     prefix)
+
+
+def toy2_plain(weights, cfg: ToyConfig, ids):
+    w = {k: v.double() for k, v in weights.items()}
+    norm = lambda x, name: x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6) * (1.0 + w[name])
+    x = w["model.embed_tokens.weight"][ids]
+    T = len(ids)
+    inv = 50.0 ** (-2.0 * torch.arange(8, dtype=torch.float64) / 16)
+    angle = torch.arange(T, dtype=torch.float64).sqrt()[:, None] * inv[None, :]
+    cos, sin = angle.cos().float().double()[:, None, :], angle.sin().float().double()[:, None, :]  # tables are 32-bit
+
+    def rotate(v):
+        a, b = v[..., :8], v[..., 8:]
+        return torch.cat([a * cos - b * sin, a * sin + b * cos], dim=-1)
+
+    for l in range(cfg.layers):
+        p = f"model.layers.{l}"
+        h = norm(x, f"{p}.input_layernorm.weight")
+        q = rotate((h @ w[f"{p}.self_attn.q_proj.weight"].T).view(T, 2, 16))
+        k = rotate((h @ w[f"{p}.self_attn.k_proj.weight"].T).view(T, 2, 16))
+        v = (h @ w[f"{p}.self_attn.v_proj.weight"].T).view(T, 2, 16)
+        a = P.attention(q, k, v, 0.25, 6).reshape(T, 32) @ w[f"{p}.self_attn.o_proj.weight"].T
+        x = x + norm(a, f"{p}.post_attention_layernorm.weight")
+        h = norm(x, f"{p}.pre_feedforward_layernorm.weight")
+        if l % 2:
+            choice = (h.float() @ weights[f"{p}.moe.router.weight"].float().T).argmax(-1)
+            f = torch.zeros_like(h)
+            for t in range(T):
+                e = int(choice[t])
+                gu = h[t] @ w[f"{p}.moe.experts.{e}.gate_up.weight"].T
+                f[t] = (torch.nn.functional.silu(gu[: cfg.hidden]) * gu[cfg.hidden:]) @ w[f"{p}.moe.experts.{e}.down.weight"].T
+        else:
+            f = (torch.nn.functional.silu(h @ w[f"{p}.mlp.gate_proj.weight"].T) * (h @ w[f"{p}.mlp.up_proj.weight"].T)) \
+                @ w[f"{p}.mlp.down_proj.weight"].T
+        x = x + norm(f, f"{p}.post_feedforward_layernorm.weight")
+    return norm(x, "model.norm.weight") @ w["model.embed_tokens.weight"].T
+
+
+def test_toy_routed_feed_forward_and_position_encoding_plug_in(tmp_path):
+    FEED_FORWARDS.register("top_one_experts", TopOneExperts, replace=True)
+    POSITION_ENCODINGS.register("root_positions", RootPositions, replace=True)
+    register_architecture(Architecture("Toy2ForCausalLM", ToyConfig.from_dict, toy2_spec, ToyConfig.to_dict), replace=True)
+    try:
+        cfg = ToyConfig("Toy2ForCausalLM", hidden=24, vocab=40, layers=4)
+        folder = write_random_model(tmp_path / "toy2", cfg, seed=11, dtype=torch.float32)
+        runner = ModelRunner.from_model_dir(folder, EngineConfig(dtype="float32", max_model_len=64, max_num_seqs=2,
+                                                                max_num_batched_tokens=64, max_prefill_chunk=64,
+                                                                max_cache_tokens=128))
+        weights = P.load_weights(folder)
+        assert any(".moe.experts.2.down.weight" in k for k in weights)  # the experts' tensors were written and read by name
+        ids = [5, 1, 33, 7, 7, 20, 39, 0, 12, 3, 18, 25, 6, 31]
+        want = toy2_plain(weights, cfg, ids)
+        runner.add_request("whole")
+        got = runner.step([("whole", ids, list(range(len(ids))))]).cpu().double()
+        assert torch.allclose(got, want, atol=1e-4)
+        # cut into portions and single tokens beside another request: the same logits
+        runner.add_request("cut")
+        parts, at = [], 0
+        for n in (3, 1, 6, 1, 3):
+            parts.append(runner.step([("cut", ids[at:at + n], list(range(n)))]).cpu().double())
+            at += n
+        assert torch.allclose(torch.cat(parts), want, atol=1e-4)
+    finally:
+        unregister_architecture("Toy2ForCausalLM")
+        FEED_FORWARDS.unregister("top_one_experts")
+        POSITION_ENCODINGS.unregister("root_positions")
