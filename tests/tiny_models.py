@@ -5,7 +5,11 @@ equal to / different from hidden), intermediate 128 / 160, vocabulary 256 (a
 power of two) / 509 (a prime), global base 1e6 / 5e5, no scaling / linear 4,
 score scalar equal to / different from the head size, eps 1e-6 / 1e-5.
 C has the head size of the large models (256), one key/value head and a
-soft-cap.
+soft-cap.  D is not tiny in its layers: two layers with the attention sizes of
+the 4B model (width 2560, heads 8:4 of 256, feed-forward 10240, window 1024,
+global scaling 8) and
+a vocabulary of 1003, for sequences that cross the window's edge; it is
+written only by the tests that use it.
 """
 
 from __future__ import annotations
@@ -82,7 +86,30 @@ CONFIG_C = {
     "final_logit_softcapping": 30.0,
 }
 
+CONFIG_D = {
+    "architectures": ["Gemma3ForCausalLM"],
+    "num_hidden_layers": 2,
+    "layer_types": ["sliding_attention", "full_attention"],
+    "hidden_size": 2560,
+    "num_attention_heads": 8,
+    "num_key_value_heads": 4,
+    "head_dim": 256,
+    "intermediate_size": 10240,
+    "vocab_size": 1003,
+    "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 8192,
+    "sliding_window": 1024,
+    "rope_theta": 1000000.0,
+    "rope_local_base_freq": 10000.0,
+    "rope_scaling": {"rope_type": "linear", "factor": 8.0},
+    "query_pre_attn_scalar": 256,
+    "hidden_activation": "gelu_pytorch_tanh",
+    "tie_word_embeddings": True,
+    "final_logit_softcapping": None,
+}
+
 CONFIGS = {"A": (CONFIG_A, 0), "B": (CONFIG_B, 1), "C": (CONFIG_C, 2)}
+LARGER = {"D": (CONFIG_D, 3)}
 
 
 def write_model(folder, name: str, dtype=torch.bfloat16, seed=None) -> Path:
@@ -92,7 +119,7 @@ def write_model(folder, name: str, dtype=torch.bfloat16, seed=None) -> Path:
     import rvllm_amd.models.gemma3  # noqa: F401  (registers the architecture)
     from rvllm_amd.weights.random_init import write_random_model
 
-    doc, default_seed = CONFIGS[name]
+    doc, default_seed = CONFIGS[name] if name in CONFIGS else LARGER[name]
     arch = architecture_of(doc)
     config = arch.read_config(doc, f"tiny config {name}")
     out = write_random_model(Path(folder), config, default_seed if seed is None else seed, dtype)
