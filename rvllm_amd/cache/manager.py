@@ -22,7 +22,7 @@ import dataclasses
 from typing import Hashable, Optional, Sequence
 
 from ..parts.base import KVNeed, StateNeed
-from .pages import CacheBookkeepingError, OutOfPages, PagePool, StateSlots
+from .pages import BlockTable, CacheBookkeepingError, OutOfPages, PagePool, StateSlots
 
 
 def group_name(window: Optional[int]) -> str:
@@ -36,7 +36,7 @@ class RequestCache:
     request: Hashable
     length: int = 0  # tokens whose keys are in the cache
     slot: int = -1
-    tables: dict = dataclasses.field(default_factory=dict)  # group -> list of pages by logical index, -1 = none
+    tables: dict = dataclasses.field(default_factory=dict)  # group -> BlockTable
 
 
 class PageGroup:
@@ -55,7 +55,7 @@ class PageGroup:
             return 0
         return max(0, length - self.window + 1) // self.page_size
 
-    def pages_to_add(self, table: list[int], new_length: int) -> int:
+    def pages_to_add(self, table, new_length: int) -> int:
         need = -(-new_length // self.page_size)
         return max(0, need - len(table))
 
@@ -91,7 +91,7 @@ class CacheManager:
     def add_request(self, request: Hashable) -> RequestCache:
         if request in self.requests:
             raise KeyError(f"request {request!r} is already live")
-        rc = RequestCache(request, 0, self.slots.take(request), {name: [] for name in self.groups})
+        rc = RequestCache(request, 0, self.slots.take(request), {name: BlockTable() for name in self.groups})
         self.requests[request] = rc
         return rc
 
@@ -106,7 +106,7 @@ class CacheManager:
         rc = self.requests.get(request)
         out = {}
         for name, g in self.groups.items():
-            table = rc.tables[name] if rc is not None else []
+            table = rc.tables[name] if rc is not None else ()
             out[name] = g.pages_to_add(table, new_length)
         return out
 
@@ -153,7 +153,7 @@ class CacheManager:
         it gets exactly the pages a request of that length holds (none behind
         a window).  For measurements on a cache filled by hand."""
         rc = self.requests[request]
-        if rc.length != 0 or any(rc.tables[name] for name in self.groups):
+        if rc.length != 0 or any(len(rc.tables[name]) for name in self.groups):
             raise ValueError("only a fresh request can adopt a length")
         plan = {}
         for name, g in self.groups.items():
@@ -163,7 +163,7 @@ class CacheManager:
                 raise OutOfPages(name, count, g.pool.free_count)
             plan[name] = (first, count)
         for name, (first, count) in plan.items():
-            rc.tables[name] = [-1] * first + self.groups[name].pool.take(request, count)
+            rc.tables[name] = BlockTable([-1] * first + self.groups[name].pool.take(request, count), passed=first)
         rc.length = length
 
     def commit(self, request: Hashable, new_length: int) -> None:
@@ -177,22 +177,19 @@ class CacheManager:
                 raise CacheBookkeepingError(f"request {request!r} committed {new_length} tokens without pages for them")
         rc.length = new_length
         for name, g in self.groups.items():
-            table = rc.tables[name]
-            passed = [i for i in range(min(g.first_kept_page(new_length), len(table))) if table[i] >= 0]
+            passed = rc.tables[name].pass_up_to(g.first_kept_page(new_length))
             if passed:
-                g.pool.give_back(request, [table[i] for i in passed])
-                for i in passed:
-                    table[i] = -1
+                g.pool.give_back(request, passed)
 
     def release(self, request: Hashable) -> None:
         """The request is finished (or set back): everything it holds returns."""
         rc = self.requests.pop(request)
         for name, g in self.groups.items():
-            g.pool.give_back(request, [p for p in rc.tables[name] if p >= 0])
+            g.pool.give_back(request, rc.tables[name].held())
         self.slots.give_back(request, rc.slot)
 
     # ---- reading -----------------------------------------------------
-    def table(self, request: Hashable, group: str) -> list[int]:
+    def table(self, request: Hashable, group: str) -> BlockTable:
         return self.requests[request].tables[group]
 
     def slot(self, request: Hashable) -> int:

@@ -11,7 +11,9 @@ the allocator is this engine's own.
 
 from __future__ import annotations
 
-from typing import Hashable, Optional
+from typing import Hashable, Iterable, Optional
+
+import numpy as np
 
 
 class OutOfPages(RuntimeError):
@@ -75,6 +77,69 @@ class PagePool:
 
 
 _NOBODY = object()
+
+
+class BlockTable:
+    """A request's pages in one group by logical index, -1 where it holds none.
+
+    Kept as an array that grows by doubling, so that a step copies a table of
+    thousands of pages into its staging buffer as one block; ``passed`` is the
+    number of leading entries that a window has already given back, so that
+    giving back looks only at what is new.  Reads like a list."""
+
+    def __init__(self, pages: Iterable[int] = (), passed: int = 0):
+        pages = list(pages)
+        self._pages = np.full(max(16, len(pages)), -1, dtype=np.int32)
+        self._pages[: len(pages)] = pages
+        self._n = len(pages)
+        self.passed = passed
+
+    def __len__(self) -> int:
+        return self._n
+
+    def __array__(self, dtype=None, copy=None):
+        view = self._pages[: self._n]
+        return view if dtype is None or dtype == view.dtype else view.astype(dtype)
+
+    def view(self) -> np.ndarray:
+        """The entries, writable, valid until the table grows."""
+        return self._pages[: self._n]
+
+    def __iter__(self):
+        return iter(self._pages[: self._n].tolist())
+
+    def __getitem__(self, index):
+        got = self._pages[: self._n][index]
+        return got.tolist() if isinstance(index, slice) else int(got)
+
+    def __eq__(self, other) -> bool:
+        return list(self) == list(other)
+
+    def extend(self, pages: Iterable[int]) -> None:
+        pages = list(pages)
+        need = self._n + len(pages)
+        if need > len(self._pages):
+            grown = np.full(max(need, 2 * len(self._pages)), -1, dtype=np.int32)
+            grown[: self._n] = self._pages[: self._n]
+            self._pages = grown
+        self._pages[self._n : need] = pages
+        self._n = need
+
+    def held(self) -> list[int]:
+        """The pages the table still names."""
+        live = self._pages[self.passed : self._n]
+        return live[live >= 0].tolist()
+
+    def pass_up_to(self, first_kept: int) -> list[int]:
+        """Forget the pages before logical index ``first_kept``; returns them."""
+        first_kept = min(first_kept, self._n)
+        if first_kept <= self.passed:
+            return []
+        gone = self._pages[self.passed : first_kept]
+        pages = gone[gone >= 0].tolist()
+        gone[:] = -1
+        self.passed = first_kept
+        return pages
 
 
 class StateSlots:

@@ -156,3 +156,39 @@ def test_random_orders_keep_the_books(seed):
         m.release(name)
     m.check()
     assert all(free == g.pool.num_pages for free, g in zip(m.free_pages().values(), m.groups.values()))
+
+
+def test_block_table_grows_and_forgets_what_a_window_passed():
+    """The array behind a table doubles as it grows; passing pages returns each
+    page once and looks only at entries that were not passed before."""
+    import numpy as np
+
+    from rvllm_amd.cache.pages import BlockTable
+
+    t = BlockTable()
+    assert len(t) == 0 and t == [] and t.held() == []
+    t.extend(range(100, 140))  # beyond the first allocation
+    assert len(t) == 40 and t[0] == 100 and t[-1] == 139 and t[38:] == [138, 139]
+    assert np.asarray(t).dtype == np.int32 and np.asarray(t).tolist() == list(range(100, 140))
+    assert t.pass_up_to(3) == [100, 101, 102] and t.passed == 3
+    assert t.pass_up_to(2) == [] and t.pass_up_to(3) == []
+    assert t.pass_up_to(5) == [103, 104] and t[:6] == [-1, -1, -1, -1, -1, 105]
+    t.extend([7])
+    assert t.held() == list(range(105, 140)) + [7]
+    assert t.pass_up_to(1000) == list(range(105, 140)) + [7] and t.held() == [] and t.passed == 41
+    adopted = BlockTable([-1, -1, 5, 6], passed=2)
+    assert adopted.held() == [5, 6] and adopted.pass_up_to(3) == [5]
+
+
+def test_commit_at_a_long_context_looks_at_new_pages_only():
+    """A window group's commit does not walk the whole table each step."""
+    m = CacheManager([KVNeed(2, 16, 8)], page_size=4, num_pages={"window8": 8}, max_requests=1)
+    m.add_request("r")
+    length = 0
+    for _ in range(300):
+        length += 3
+        m.extend("r", length)
+        m.commit("r", length)
+        m.check()
+    table = m.table("r", "window8")
+    assert table.passed == m.groups["window8"].first_kept_page(length) and len(table.held()) <= 4
