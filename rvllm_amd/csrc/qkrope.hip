@@ -108,6 +108,60 @@ __device__ __forceinline__ void qkr_load(const void* qkv, int slices, long long 
     if (lane + j * RV_WAVE >= half) lo[j] = hi[j] = 0.f;
 }
 
+// The values of a step's tokens, written a page at a time.  Values lie
+// transposed inside a page (kv_layout.h), so a wave per token and head
+// scatters them two or four bytes at a time; for prompt portions that is most
+// of such a kernel's time.  Here a block takes one page of one request and one
+// key/value head: thread d gathers the page's tokens at dimension d (for a
+// fixed token the threads read one contiguous row) and writes row d of the
+// page, 16 bytes at a time when the portion covers the whole page.  The
+// kernels below give the blocks of extra rows of their grid to this work
+// (`write_kv` 2), so that a prompt step writes keys and values in one launch.
+struct ValuePages {
+  const int* q_start;      // [requests + 1]
+  const int* chunk_start;  // [requests]: position of each portion's first token
+  int num_requests;
+  int pages_per_request;   // a portion of n tokens touches at most (n - 1) / page_size + 2 pages
+};
+
+template <typename T>
+__device__ void v_write_page(long long unit, const ValuePages& V, const T* __restrict__ qkv, T* __restrict__ v_pages,
+                             const int* __restrict__ block_table, int table_width, int page_size, int num_pages,
+                             int nq, int nkv, int hd) {
+  if (unit >= (long long)V.pages_per_request * nkv * V.num_requests) return;
+  const int rel = (int)(unit % V.pages_per_request);
+  const int kvh = (int)(unit / V.pages_per_request % nkv);
+  const int b = (int)(unit / V.pages_per_request / nkv);
+  const int q0 = V.q_start[b];
+  const int n = V.q_start[b + 1] - q0;
+  const int s = V.chunk_start[b];
+  if (n <= 0) return;
+  const int lp = s / page_size + rel;
+  const int lo = s > lp * page_size ? s : lp * page_size;
+  const int hi = s + n < (lp + 1) * page_size ? s + n : (lp + 1) * page_size;
+  if (lo >= hi || lp >= table_width) return;
+  const int page = block_table[(size_t)b * table_width + lp];
+  if (page < 0 || page >= num_pages) return;
+  const size_t width = (size_t)(nq + 2 * nkv) * hd;
+  const T* src = qkv + (size_t)(q0 + lo - s) * width + (size_t)(nq + nkv + kvh) * hd;  // token at position lo
+  const int slot0 = lo - lp * page_size;
+  constexpr int VEC = 16 / sizeof(T);  // elements of a 16-byte store
+  const bool whole = hi - lo == page_size && page_size % VEC == 0;
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    T* row = v_pages + rv_v_index(page, kvh, 0, d, nkv, page_size, hd);
+    if (whole) {
+      for (int g = 0; g < page_size; g += VEC) {
+        T v[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = src[(size_t)(g + i) * width + d];
+        *(uint4*)(row + g) = *(const uint4*)v;
+      }
+    } else {
+      for (int i = 0; i < hi - lo; ++i) row[slot0 + i] = src[(size_t)i * width + d];
+    }
+  }
+}
+
 template <typename T>
 __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int slices, long long slice_stride,
                                              T* __restrict__ q_out,
@@ -117,9 +171,15 @@ __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int s
                                              const int* __restrict__ positions, const int* __restrict__ token_req,
                                              const int* __restrict__ block_table, int table_width,
                                              T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size,
-                                             int num_pages, int nq, int nkv, int hd, int write_kv) {
+                                             int num_pages, int nq, int nkv, int hd, int write_kv, ValuePages V) {
   const int wave = threadIdx.x / RV_WAVE;
   const int lane = threadIdx.x & (RV_WAVE - 1);
+  const int head_rows = ((write_kv == 1 ? nq + 2 * nkv : nq + nkv) + 3) / 4;
+  if ((int)blockIdx.y >= head_rows) {  // the rows of the grid beyond the heads write values a page at a time
+    v_write_page<T>((long long)(blockIdx.y - head_rows) * gridDim.x + blockIdx.x, V, (const T*)qkv, v_pages, block_table,
+                    table_width, page_size, num_pages, nq, nkv, hd);
+    return;
+  }
   const int t = blockIdx.x;
   const int head = blockIdx.y * 4 + wave;
   const int total_heads = nq + 2 * nkv;
@@ -167,7 +227,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int s
     if (is_k) {
       dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
     } else {
-      if (write_kv == 2) return;  // values are written a page at a time by v_write_pages_kernel
+      if (write_kv == 2) return;  // values are written a page at a time by other blocks of this launch
       // values are stored as projected, transposed inside the page
       T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
 #pragma unroll
@@ -245,9 +305,15 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
                                                  int rot, const int* __restrict__ positions,
                                                  const int* __restrict__ token_req, const int* __restrict__ block_table,
                                                  int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                                 int page_size, int num_pages, int nq, int nkv, int hd, int write_kv) {
+                                                 int page_size, int num_pages, int nq, int nkv, int hd, int write_kv, ValuePages V) {
   const int wave = threadIdx.x / RV_WAVE;
   const int lane = threadIdx.x & (RV_WAVE - 1);
+  const int head_rows = ((write_kv == 1 ? nq + 2 * nkv : nq + nkv) + 3) / 4;
+  if ((int)blockIdx.y >= head_rows) {  // the rows of the grid beyond the heads write values a page at a time
+    v_write_page<T>((long long)(blockIdx.y - head_rows) * gridDim.x + blockIdx.x, V, (const T*)qkv, v_pages, block_table,
+                    table_width, page_size, num_pages, nq, nkv, hd);
+    return;
+  }
   const int t = blockIdx.x;
   const int head = blockIdx.y * 4 + wave;
   const int total_heads = nq + 2 * nkv;
@@ -315,7 +381,7 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
     if (is_k) {
       dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
     } else {
-      if (write_kv == 2) return;  // values are written a page at a time by v_write_pages_kernel
+      if (write_kv == 2) return;  // values are written a page at a time by other blocks of this launch
       // values are stored as projected, transposed inside the page
       T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
       if (active) {
@@ -346,73 +412,6 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
   if (active) QkrVec<T>::store(dst + d0, x);
 }
 
-// The values of a step's tokens, written a page at a time.  Values lie
-// transposed inside a page (kv_layout.h), so the kernels above, a wave per
-// token and head, scatter them two or four bytes at a time; for prompt
-// portions that is most of their time.  Here a block takes one page of one
-// request and one key/value head: thread d gathers the page's tokens at
-// dimension d (for a fixed token the threads read one contiguous row) and writes
-// row d of the page, 16 bytes at a time when the portion covers the whole page.
-// grid (pages a portion may touch, kv heads, requests).
-template <typename T>
-__global__ void __launch_bounds__(256)
-v_write_pages_kernel(const T* __restrict__ qkv, T* __restrict__ v_pages, const int* __restrict__ q_start,
-                     const int* __restrict__ chunk_start, const int* __restrict__ block_table, int table_width,
-                     int page_size, int num_pages, int nq, int nkv, int hd) {
-  const int b = blockIdx.z, kvh = blockIdx.y;
-  const int q0 = q_start[b];
-  const int n = q_start[b + 1] - q0;
-  const int s = chunk_start[b];
-  if (n <= 0) return;
-  const int lp = s / page_size + blockIdx.x;
-  const int lo = s > lp * page_size ? s : lp * page_size;
-  const int hi = s + n < (lp + 1) * page_size ? s + n : (lp + 1) * page_size;
-  if (lo >= hi || lp >= table_width) return;
-  const int page = block_table[(size_t)b * table_width + lp];
-  if (page < 0 || page >= num_pages) return;
-  const size_t width = (size_t)(nq + 2 * nkv) * hd;
-  const T* src = qkv + (size_t)(q0 + lo - s) * width + (size_t)(nq + nkv + kvh) * hd;  // token at position lo
-  const int slot0 = lo - lp * page_size;
-  constexpr int VEC = 16 / sizeof(T);  // elements of a 16-byte store
-  const bool whole = hi - lo == page_size && page_size % VEC == 0;
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    T* row = v_pages + rv_v_index(page, kvh, 0, d, nkv, page_size, hd);
-    if (whole) {
-      for (int g = 0; g < page_size; g += VEC) {
-        T v[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) v[i] = src[(size_t)(g + i) * width + d];
-        *(uint4*)(row + g) = *(const uint4*)v;
-      }
-    } else {
-      for (int i = 0; i < hi - lo; ++i) row[slot0 + i] = src[(size_t)i * width + d];
-    }
-  }
-}
-
-extern "C" int rv_v_write_pages(hipStream_t stream, const void* qkv, void* v_pages, const int* q_start,
-                                const int* chunk_start, const int* block_table, int table_width, int page_size,
-                                int num_pages, int dtype, int num_requests, int max_portion, int nq, int nkv, int hd) {
-  RV_CHECK(num_requests >= 0 && max_portion >= 1 && nq > 0 && nkv > 0 && hd > 0, "v_write_pages: bad sizes");
-  RV_CHECK(page_size > 0 && num_pages > 0 && table_width > 0 && qkv && v_pages && q_start && chunk_start && block_table,
-           "v_write_pages: needs the projection's output, the pages and the step's tables");
-  RV_CHECK(num_requests <= 65535 && nkv <= 65535, "v_write_pages: too many requests or heads for one launch");
-  if (num_requests == 0) return 0;
-  // a portion of n tokens touches at most (n - 1) / page_size + 2 pages
-  dim3 grid((max_portion - 1) / page_size + 2, nkv, num_requests);
-  if (dtype == RV_F32)
-    v_write_pages_kernel<float><<<grid, dim3(256), 0, stream>>>((const float*)qkv, (float*)v_pages, q_start, chunk_start,
-                                                               block_table, table_width, page_size, num_pages, nq, nkv, hd);
-  else if (dtype == RV_BF16)
-    v_write_pages_kernel<bf16_t><<<grid, dim3(256), 0, stream>>>((const bf16_t*)qkv, (bf16_t*)v_pages, q_start,
-                                                                chunk_start, block_table, table_width, page_size,
-                                                                num_pages, nq, nkv, hd);
-  else
-    return rv_fail("v_write_pages: unsupported dtype %d", dtype);
-  RV_LAUNCH_CHECK("v_write_pages");
-  return 0;
-}
-
 // `slices` 0: qkv holds T values [tokens, (nq + 2 nkv) * hd]; otherwise 32-bit
 // partial sums [slices][tokens][...], slice_stride elements apart.
 extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int slices, long long slice_stride,
@@ -420,7 +419,8 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
                                         const void* k_w, int w_f32, float eps, float offset, const float* rope_cos,
                                         const float* rope_sin, int rot, const int* positions, const int* token_req, const int* block_table,
                                         int table_width, void* k_pages, void* v_pages, int page_size, int num_pages,
-                                        int dtype, int num_tokens, int nq, int nkv, int hd, int write_kv) {
+                                        int dtype, int num_tokens, int nq, int nkv, int hd, int write_kv,
+                                        const int* q_start, const int* chunk_start, int num_requests, int max_portion) {
   RV_CHECK(num_tokens >= 0 && nq > 0 && nkv > 0, "qk_norm_rope: bad sizes T=%d nq=%d nkv=%d", num_tokens, nq, nkv);
   RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= (long long)num_tokens * (nq + 2 * nkv) * hd),
            "qk_norm_rope: bad partial sums");
@@ -432,20 +432,32 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
   RV_CHECK(!write_kv || (page_size > 0 && num_pages > 0 && table_width > 0 && block_table && k_pages && v_pages),
            "qk_norm_rope: cache write needs pages and a block table");
   if (num_tokens == 0) return 0;
-  // write_kv 0: nothing goes to the cache; 1: keys and values; 2: keys only (values by rv_v_write_pages)
+  // write_kv 0: nothing goes to the cache; 1: keys and values, token by token; 2: keys token by token and values
+  // a page at a time, by extra rows of blocks (for prompt portions; needs the step's portions and whole values,
+  // not partial sums)
   RV_CHECK(write_kv >= 0 && write_kv <= 2, "qk_norm_rope: write_kv is 0, 1 or 2");
-  dim3 grid(num_tokens, rv_div_up(write_kv == 1 ? nq + 2 * nkv : nq + nkv, 4)), block(4 * RV_WAVE);
+  ValuePages V = {q_start, chunk_start, num_requests, 0};
+  int rows = rv_div_up(write_kv == 1 ? nq + 2 * nkv : nq + nkv, 4);
+  if (write_kv == 2) {
+    RV_CHECK(slices == 0 && q_start && chunk_start && num_requests >= 1 && max_portion >= 1,
+             "qk_norm_rope: values by pages need the step's portions and a projection that is already added up");
+    V.pages_per_request = (max_portion - 1) / page_size + 2;
+    const long long units = (long long)V.pages_per_request * nkv * num_requests;
+    rows += (int)((units + num_tokens - 1) / num_tokens);
+    RV_CHECK(rows <= 65535, "qk_norm_rope: too many pages of values for one launch");
+  }
+  dim3 grid(num_tokens, rows), block(4 * RV_WAVE);
   if (hd % 8 == 0 && hd <= 4 * RV_WAVE && rot % 8 == 0) {  // four dimensions a lane
     if (dtype == RV_F32)
       qk_norm_rope_kv_write_vec_kernel<float><<<grid, block, 0, stream>>>(
           qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions,
           token_req, block_table, table_width, (float*)k_pages, (float*)v_pages, page_size, num_pages, nq, nkv, hd,
-          write_kv);
+          write_kv, V);
     else if (dtype == RV_BF16)
       qk_norm_rope_kv_write_vec_kernel<bf16_t><<<grid, block, 0, stream>>>(
           qkv, slices, slice_stride, (bf16_t*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions,
           token_req, block_table, table_width, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, num_pages, nq, nkv, hd,
-          write_kv);
+          write_kv, V);
     else
       return rv_fail("qk_norm_rope: unsupported dtype %d", dtype);
     RV_LAUNCH_CHECK("qk_norm_rope_kv_write");
@@ -454,11 +466,11 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
   if (dtype == RV_F32)
     qk_norm_rope_kv_write_kernel<float><<<grid, block, 0, stream>>>(
         qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions, token_req,
-        block_table, table_width, (float*)k_pages, (float*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv);
+        block_table, table_width, (float*)k_pages, (float*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv, V);
   else if (dtype == RV_BF16)
     qk_norm_rope_kv_write_kernel<bf16_t><<<grid, block, 0, stream>>>(
         qkv, slices, slice_stride, (bf16_t*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions, token_req,
-        block_table, table_width, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv);
+        block_table, table_width, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv, V);
   else
     return rv_fail("qk_norm_rope: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("qk_norm_rope_kv_write");

@@ -263,9 +263,11 @@ def qk_norm_rope_kv_write(qkv, q_out: torch.Tensor, q_weight: Optional[torch.Ten
                           token_req: torch.Tensor, block_table: Optional[torch.Tensor],
                           k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], num_q_heads: int,
                           num_kv_heads: int, head_dim: int, write_kv: bool = True,
-                          values_by_page: bool = False) -> torch.Tensor:
+                          values_by_page=None) -> torch.Tensor:
     """Query/key norm and rotation; queries to ``q_out``, keys and values into the cache (``write_kv``).
-    With ``values_by_page`` the values are left to ``v_write_pages``."""
+    ``values_by_page`` is the step (its q_start, chunk_start, num_requests, max_portion) when extra blocks of the
+    same launch are to write the values a page at a time, which pays for prompt portions; the projection must
+    then be whole, not partial sums."""
     qptr, slices, stride, n, qkv_width, qkv_dtype = _branch_args(qkv, "qk_norm_rope")
     rope_cos, rope_sin = rope if rope is not None else (None, None)
     _gpu(q_out, q_weight, k_weight, rope_cos, rope_sin, positions, token_req, block_table, k_pages, v_pages)
@@ -284,6 +286,11 @@ def qk_norm_rope_kv_write(qkv, q_out: torch.Tensor, q_weight: Optional[torch.Ten
             _need(table.dtype == torch.float32 and table.is_contiguous() and table.shape == (n, rotary_dim // 2),
                   f"qk_norm_rope: the table of cosines and sines must be 32-bit [{n}, {rotary_dim // 2}]")
     page_size = num_pages = width = 0
+    by_page = bool(write_kv) and values_by_page is not None
+    if by_page:
+        _need(slices == 0, "qk_norm_rope: values by pages need a projection that is already added up")
+        _gpu(values_by_page.q_start, values_by_page.chunk_start)
+        _i32(values_by_page.q_start, values_by_page.chunk_start)
     if write_kv:
         _need(k_pages is not None and v_pages is not None and block_table is not None, "qk_norm_rope: no cache given")
         _i32(block_table)
@@ -297,28 +304,14 @@ def qk_norm_rope_kv_write(qkv, q_out: torch.Tensor, q_weight: Optional[torch.Ten
         _c_float(offset), _ptr(rope_cos), _ptr(rope_sin), _c_int(rotary_dim if rope is not None else 0), _ptr(positions),
         _ptr(token_req), _ptr(block_table), _c_int(width), _ptr(k_pages), _ptr(v_pages), _c_int(page_size),
         _c_int(num_pages), _dt(q_out), _c_int(n), _c_int(num_q_heads), _c_int(num_kv_heads), _c_int(head_dim),
-        _c_int((2 if values_by_page else 1) if write_kv else 0)))
+        _c_int((2 if by_page else 1) if write_kv else 0),
+        _ptr(values_by_page.q_start if by_page else None), _ptr(values_by_page.chunk_start if by_page else None),
+        _c_int(values_by_page.num_requests if by_page else 0), _c_int(values_by_page.max_portion if by_page else 0)))
     return q_out
 
 
 # Portions of at least this many tokens have their values written a page at a time.
 VALUES_BY_PAGE_MIN_PORTION = 16
-
-
-def v_write_pages(qkv: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, step, num_q_heads: int,
-                  num_kv_heads: int, head_dim: int) -> None:
-    """The values of the step's tokens into their pages, a page of a request and a key/value head per block
-    (whole pages in 16-byte stores): for steps with prompt portions."""
-    _gpu(qkv, v_pages, block_table, step.q_start, step.chunk_start)
-    _i32(block_table, step.q_start, step.chunk_start)
-    num_pages, nkv, hd, page_size = v_pages.shape
-    _need((nkv, hd) == (num_kv_heads, head_dim), "v_write_pages: cache pages do not fit the heads")
-    _need(qkv.dim() == 2 and qkv.shape[1] == (num_q_heads + 2 * num_kv_heads) * head_dim and qkv.dtype == v_pages.dtype,
-          "v_write_pages: bad qkv")
-    _check(library().rv_v_write_pages(
-        _stream(), _ptr(qkv), _ptr(v_pages), _ptr(step.q_start), _ptr(step.chunk_start), _ptr(block_table),
-        _c_int(block_table.shape[1]), _c_int(page_size), _c_int(num_pages), _dt(qkv), _c_int(step.num_requests),
-        _c_int(step.max_portion), _c_int(num_q_heads), _c_int(num_kv_heads), _c_int(head_dim)))
 
 
 def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,

@@ -80,16 +80,15 @@ class PagedAttention(Mixer):
         q = torch.empty((n, self.q_size), dtype=x.dtype, device=x.device)
         table = step.block_tables[cache.group]
         norm = self.qk_norm or {}
-        # prompt portions: values go into their pages a page at a time, in wide stores
+        # prompt portions: values go into their pages a page at a time, in wide stores, by blocks of the same launch
         by_page = (cache.writes and isinstance(qkv, torch.Tensor)
                    and step.max_portion >= ops.VALUES_BY_PAGE_MIN_PORTION)
         ops.qk_norm_rope_kv_write(
             qkv, q, self.q_norm_w, self.k_norm_w, float(norm.get("eps", 0.0)),
             1.0 if norm.get("unit_offset", False) else 0.0, self.position.tables(step),
             self.position.rotary_dim, step.positions, step.token_req, table, cache.k_pages, cache.v_pages,
-            self.num_heads, self.num_kv_heads, self.head_dim, write_kv=cache.writes, values_by_page=by_page)
-        if by_page:
-            ops.v_write_pages(qkv, cache.v_pages, table, step, self.num_heads, self.num_kv_heads, self.head_dim)
+            self.num_heads, self.num_kv_heads, self.head_dim, write_kv=cache.writes,
+            values_by_page=step if by_page else None)
         attn = torch.empty_like(q)
         ops.paged_attention(q, cache.k_pages, cache.v_pages, table, step, attn, self.num_heads, self.scale,
                             self.window)
