@@ -435,6 +435,17 @@ def test_paged_attention_shared_tiles_long_prompt_portions():
         assert torch.allclose(case.run("mfma", 1.0 / 16).float(), want, **tol(torch.bfloat16)), (portions, window)
 
 
+@pytest.mark.parametrize("nq,nkv,hd,page_size", [(8, 4, 256, 16), (6, 2, 64, 64)])
+def test_paged_attention_shared_tiles_beyond_the_table_kept_in_lds(nq, nkv, hd, page_size):
+    """Portions deep in a long context: the kernel keeps the table entries of 8192 keys at hand and has to fetch
+    more of the table on its way, once and twice; with a window it starts far from the table's beginning."""
+    for portions, window in (([(8200, 40), (16500, 33)], None), ([(9000, 64)], 1024)):
+        case = Case(portions, nq, nkv, hd, page_size, torch.bfloat16, 21, window)
+        want = case.reference(hd ** -0.5).float()
+        got = case.run("mfma", hd ** -0.5, prefill_kernel=True).float()
+        assert torch.allclose(got, want, **tol(torch.bfloat16)), (portions, window)
+
+
 def _plant(case, b, key, head, dim, value):
     """Key `key` of request b becomes `value` at one dimension and nothing else, in the log and in the pages."""
     k = case.k_all[b]
