@@ -338,11 +338,14 @@ extern "C" int rv_add_rmsnorm(hipStream_t stream, const void* branch, int slices
 }
 
 // ---------------------------------------------------------------------------
-// gated activation: out[t,i] = act(gu[t,i]) * gu[t,I+i]
+// gated activation: out[t,i] = act(gate[t,i]) * up[t,i]
 // act 0: gelu, tanh form; act 1: silu
+// The two lie in one row of gu: halves (gates, then ups: gate i at i, up i at
+// I + i) or, FOURS, as a product against weight rows in fours leaves them (two
+// gates, then their two ups: gate i at 4 (i / 2) + i % 2, up i two further).
 // ---------------------------------------------------------------------------
 
-template <typename T, int V, int ACT>
+template <typename T, int V, int ACT, bool FOURS>
 __global__ void gated_act_kernel(const void* __restrict__ gu, int slices, long long slice_stride, T* __restrict__ out,
                                  int inter, long long groups_total) {
   const long long gidx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -350,10 +353,23 @@ __global__ void gated_act_kernel(const void* __restrict__ gu, int slices, long l
   const int groups_per_row = inter / V;
   const long long t = gidx / groups_per_row;
   const int i = (int)(gidx - t * groups_per_row) * V;
-  const size_t at = (size_t)t * 2 * inter + i;
   float g[V], u[V];
-  row_load_branch<T, V>(gu, slices, slice_stride, at, g);
-  row_load_branch<T, V>(gu, slices, slice_stride, at + inter, u);
+  if constexpr (FOURS) {  // V is a multiple of 4 here: the thread's outputs are its 2 V neighbouring values
+    const size_t at = (size_t)t * 2 * inter + 2 * (size_t)i;
+    float a[V], b[V];
+    row_load_branch<T, V>(gu, slices, slice_stride, at, a);
+    row_load_branch<T, V>(gu, slices, slice_stride, at + V, b);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const int at4 = 4 * (v / 2) + v % 2;  // among the 2 V values
+      g[v] = at4 < V ? a[at4] : b[at4 - V];
+      u[v] = at4 + 2 < V ? a[at4 + 2] : b[at4 + 2 - V];
+    }
+  } else {
+    const size_t at = (size_t)t * 2 * inter + i;
+    row_load_branch<T, V>(gu, slices, slice_stride, at, g);
+    row_load_branch<T, V>(gu, slices, slice_stride, at + inter, u);
+  }
 #pragma unroll
   for (int v = 0; v < V; ++v) g[v] = rv_gated<T, ACT>(g[v], u[v]);
   row_store<T, V>(out + (size_t)t * inter + i, g);
@@ -362,30 +378,38 @@ __global__ void gated_act_kernel(const void* __restrict__ gu, int slices, long l
 // `slices` 0: gu holds T values [rows, 2*inter]; otherwise 32-bit partial sums
 // [slices][rows][2*inter], slice_stride elements apart.
 extern "C" int rv_gated_act(hipStream_t stream, const void* gu, int slices, long long slice_stride, void* out,
-                            int dtype, int rows, int inter, int act) {
+                            int dtype, int rows, int inter, int act, int fours) {
   RV_CHECK(rows >= 0 && inter > 0, "gated_act: bad sizes rows=%d inter=%d", rows, inter);
   RV_CHECK(act == 0 || act == 1, "gated_act: unknown activation %d", act);
+  RV_CHECK(!fours || inter % 4 == 0, "gated_act: rows in fours need a width that is a multiple of 4, got %d", inter);
   RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= 2ll * rows * inter), "gated_act: bad partial sums");
   if (rows == 0) return 0;
-#define RV_GA(T, V, A)                                                                                       \
-  do {                                                                                                       \
-    const long long groups = (long long)rows * (inter / V);                                                  \
-    gated_act_kernel<T, V, A><<<dim3(rv_div_up(groups, 256)), dim3(256), 0, stream>>>(gu, slices, slice_stride, \
-                                                                                     (T*)out, inter, groups); \
+#define RV_GA(T, V, A, F)                                                                                          \
+  do {                                                                                                             \
+    const long long groups = (long long)rows * (inter / V);                                                        \
+    gated_act_kernel<T, V, A, F><<<dim3(rv_div_up(groups, 256)), dim3(256), 0, stream>>>(gu, slices, slice_stride, \
+                                                                                        (T*)out, inter, groups);   \
   } while (0)
-#define RV_GA_T(T)                                     \
-  do {                                                 \
-    constexpr int VV = RowVec<T>::V;                   \
-    if (inter % VV == 0) {                             \
-      if (act == 0) RV_GA(T, VV, 0); else RV_GA(T, VV, 1); \
-    } else {                                           \
-      if (act == 0) RV_GA(T, 1, 0); else RV_GA(T, 1, 1);   \
-    }                                                  \
+#define RV_GA_A(T, V, F)                              \
+  do {                                                \
+    if (act == 0) RV_GA(T, V, 0, F); else RV_GA(T, V, 1, F); \
+  } while (0)
+#define RV_GA_T(T)                                                       \
+  do {                                                                   \
+    constexpr int VV = RowVec<T>::V; /* a multiple of 4 */               \
+    if (fours) {                                                         \
+      if (inter % VV != 0)                                               \
+        return rv_fail("gated_act: rows in fours need a width that is a multiple of %d, got %d", VV, inter); \
+      RV_GA_A(T, VV, true);                                              \
+    } else {                                                             \
+      if (inter % VV == 0) RV_GA_A(T, VV, false); else RV_GA_A(T, 1, false); \
+    }                                                                    \
   } while (0)
   if (dtype == RV_F32) RV_GA_T(float);
   else if (dtype == RV_BF16) RV_GA_T(bf16_t);
   else return rv_fail("gated_act: unsupported dtype %d", dtype);
 #undef RV_GA_T
+#undef RV_GA_A
 #undef RV_GA
   RV_LAUNCH_CHECK("gated_act");
   return 0;

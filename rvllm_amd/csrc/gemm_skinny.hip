@@ -57,11 +57,12 @@ __device__ __forceinline__ void sk_store1<uint16_t>(uint16_t* p, float a) {
 
 // grid (row blocks, K slices); block = waves x 64.  With one slice the result
 // goes to `out` as TC; with more, slice s writes 32-bit sums to part[s][M][N].
-// ACT < 0: x is [M, K].  ACT 0 or 1: x is [M, 2K], the gates beside the ups as
-// the product before left them, and what is multiplied is act(gate) * up,
-// worked out while a piece of x is staged (rounded to bf16 there, exactly as
-// the separate kernel for it would store it): a kernel and a pass over memory
-// less.  Every block of rows repeats that work, so it pays for few rows only.
+// ACT 0 or 1: W holds the rows of a gate and an up projection in fours, two
+// gates and then their two ups; a lane's four sums are then two gates and
+// their ups, and what an unsliced product stores is act(gate) * up, N / 2
+// values a row (the sums rounded to bf16 first, exactly as the separate kernel
+// for it would read them): a kernel and a pass over memory less, at no cost.
+// A sliced product stores its partial sums as for ACT < 0.
 template <int MT, typename TC, int ACT = -1>
 __global__ void __launch_bounds__(SK_MAX_WAVES * 64)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, TC* __restrict__ out,
@@ -94,7 +95,6 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   // a thread holds at most PIECES / 256 pieces (blocks have at least 4 waves)
   constexpr int MAX_REGS = (PIECES + 255) / 256;
   uint4 staged[MAX_REGS];
-  uint4 staged_up[ACT >= 0 ? MAX_REGS : 1];
   const int last_k = kend - 8;  // the last 16-byte piece of this slice (slices are multiples of 8 long)
   auto stage_load = [&](int c) {
 #pragma unroll
@@ -106,7 +106,6 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
       m = m < M ? m : M - 1;
       k = k < last_k ? k : last_k;
       staged[n] = *(const uint4*)(x + (size_t)m * ldx + k);
-      if constexpr (ACT >= 0) staged_up[n] = *(const uint4*)(x + (size_t)m * ldx + K + k);
     }
   };
   auto stage_store = [&](int c, int buf) {
@@ -124,19 +123,6 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
       // The staged values count as used only from here on: otherwise the masking
       // drifts up between the products, and its wait for x drains the ring.
       asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
-      if (ACT >= 0 && m < M) {  // rows past M are never stored: no activation for them
-        uint4 u = staged_up[n];
-        asm volatile("" : "+v"(u.x), "+v"(u.y), "+v"(u.z), "+v"(u.w));
-        const uint32_t gw[4] = {v.x, v.y, v.z, v.w}, uw[4] = {u.x, u.y, u.z, u.w};
-        uint32_t r[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float lo = rv_gated<bf16_t, ACT>(__uint_as_float(gw[i] << 16), __uint_as_float(uw[i] << 16));
-          const float hi = rv_gated<bf16_t, ACT>(__uint_as_float(gw[i] & 0xffff0000u), __uint_as_float(uw[i] & 0xffff0000u));
-          r[i] = rv_pack_bf16x2(lo, hi);
-        }
-        v = make_uint4(r[0], r[1], r[2], r[3]);
-      }
       v.x &= keep, v.y &= keep, v.z &= keep, v.w &= keep;
       *(uint4*)(&xs[buf][m][col]) = v;
     }
@@ -206,6 +192,13 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         if (nb + i < N) o[i] = acc[mt][i];
+    } else if constexpr (ACT >= 0) {
+      if (nb < N) {  // N is a multiple of 4
+        auto as_stored = [](float v) { return __uint_as_float((uint32_t)rv_f32_to_bf16_bits(v) << 16); };
+        TC* o = out + (size_t)m * ldc + nb / 2;
+        sk_store1<TC>(o, rv_gated<bf16_t, ACT>(as_stored(acc[mt][0]), as_stored(acc[mt][2])));
+        sk_store1<TC>(o + 1, rv_gated<bf16_t, ACT>(as_stored(acc[mt][1]), as_stored(acc[mt][3])));
+      }
     } else {
       TC* o = out + (size_t)m * ldc + nb;
 #pragma unroll
@@ -343,26 +336,40 @@ extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, 
   return rv_fail("gemm_skinny: unsupported output dtype %d", out_dtype);
 }
 
-// The product of act(gate) * up with W: x is [M, 2K] (gates, then ups), M at most 16.
-// act 0: gelu in its tanh form, 1: silu.  Otherwise as rv_gemm_skinny.
-extern "C" int rv_gemm_skinny_gated(hipStream_t stream, const void* x, const void* w, void* out, int out_dtype,
-                                    float* part, int M, int N, int K, long long ldx, long long ldw, long long ldc,
-                                    int do_reduce, int act) {
-  RV_CHECK(M >= 0 && M <= 16 && N > 0 && K > 0, "gemm_skinny_gated: M=%d must be at most 16 (N=%d K=%d)", M, N, K);
-  RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny_gated: K and the row strides must be multiples of 8");
-  RV_CHECK(ldx >= 2ll * K && ldw >= K && ldc >= N, "gemm_skinny_gated: leading dimensions too small");
-  RV_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny_gated: operands must be 16-byte aligned");
-  RV_CHECK(act == 0 || act == 1, "gemm_skinny_gated: unknown activation %d", act);
+// act(x W_gate^T) * (x W_up^T) in one kernel: W [N, K] holds the rows of the two projections in fours (gates
+// 2q, 2q + 1, then ups 2q, 2q + 1), `out` is [M, N / 2].  Only for shapes whose plan has one slice
+// (rv_gemm_skinny_slices); act 0: gelu in its tanh form, 1: silu.  Otherwise as rv_gemm_skinny.
+extern "C" int rv_gemm_skinny_gate_up(hipStream_t stream, const void* x, const void* w, void* out, int out_dtype,
+                                      int M, int N, int K, long long ldx, long long ldw, long long ldc, int act) {
+  RV_CHECK(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_gate_up: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
+  RV_CHECK(N % 4 == 0, "gemm_skinny_gate_up: N=%d must be a multiple of 4 (two gates, two ups)", N);
+  RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny_gate_up: K and the row strides must be multiples of 8");
+  RV_CHECK(ldx >= K && ldw >= K && ldc >= N / 2, "gemm_skinny_gate_up: leading dimensions too small");
+  RV_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny_gate_up: operands must be 16-byte aligned");
+  RV_CHECK(act == 0 || act == 1, "gemm_skinny_gate_up: unknown activation %d", act);
+  RV_CHECK(rv_gemm_skinny_slices(N, K) == 1, "gemm_skinny_gate_up: the plan for N=%d K=%d has slices", N, K);
   if (M == 0) return 0;
+  const int mt = rv_div_up(M, 16);
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
-  if (out_dtype == RV_F32)
-    return act == 0 ? sk_launch<1, float, 0>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc, do_reduce)
-                    : sk_launch<1, float, 1>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc, do_reduce);
-  if (out_dtype == RV_BF16)
-    return act == 0 ? sk_launch<1, uint16_t, 0>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc, do_reduce)
-                    : sk_launch<1, uint16_t, 1>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc, do_reduce);
-  return rv_fail("gemm_skinny_gated: unsupported output dtype %d", out_dtype);
+#define SK_CASE(MTV)                                                                                                \
+  case MTV:                                                                                                         \
+    if (out_dtype == RV_F32)                                                                                        \
+      return act == 0 ? sk_launch<MTV, float, 0>(stream, xp, wp, (float*)out, nullptr, M, N, K, ldx, ldw, ldc, 1)   \
+                      : sk_launch<MTV, float, 1>(stream, xp, wp, (float*)out, nullptr, M, N, K, ldx, ldw, ldc, 1);  \
+    if (out_dtype == RV_BF16)                                                                                       \
+      return act == 0                                                                                               \
+                 ? sk_launch<MTV, uint16_t, 0>(stream, xp, wp, (uint16_t*)out, nullptr, M, N, K, ldx, ldw, ldc, 1)  \
+                 : sk_launch<MTV, uint16_t, 1>(stream, xp, wp, (uint16_t*)out, nullptr, M, N, K, ldx, ldw, ldc, 1); \
+    break;
+  switch (mt) {
+    SK_CASE(1)
+    SK_CASE(2)
+    SK_CASE(3)
+    SK_CASE(4)
+  }
+#undef SK_CASE
+  return rv_fail("gemm_skinny_gate_up: unsupported output dtype %d", out_dtype);
 }
 
 // out[m][n] (bf16 or 32-bit) = sum over slices of part[s][m][n].

@@ -205,8 +205,26 @@ def add_rmsnorm(branch, weight: torch.Tensor, eps: float, offset: float, residua
 ACTIVATIONS = {"gelu_pytorch_tanh": 0, "gelu_tanh": 0, "silu": 1}
 
 
-def gated_act(gate_up, activation: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]; ``gate_up`` is a tensor or ``SlicedSums``."""
+# The widths whose gate and up rows may lie in fours (see ``rows_in_fours``): a thread of ``gated_act`` then takes
+# its 16 bytes of outputs from 32 neighbouring bytes.
+FOURS_WIDTH_MULTIPLE = 8
+
+
+def rows_in_fours(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """The rows of a gate and an up projection ``[I, H]`` as one matrix ``[2 I, H]`` in fours: gates 2q and
+    2q + 1, then ups 2q and 2q + 1.  A product against it leaves each gate two places from its up, so that
+    ``gemm_bf16_gate_up`` can apply the activation where it holds the sums, and ``gated_act(..., fours=True)``
+    reads both from neighbouring bytes."""
+    inter, hidden = gate.shape
+    _need(up.shape == gate.shape and inter % 2 == 0, "rows_in_fours: two matrices of one shape with an even number of rows")
+    return torch.cat([gate.reshape(inter // 2, 2, hidden), up.reshape(inter // 2, 2, hidden)], dim=1).reshape(
+        2 * inter, hidden).contiguous()
+
+
+def gated_act(gate_up, activation: str, out: Optional[torch.Tensor] = None, fours: bool = False) -> torch.Tensor:
+    """out[t, i] = act(gate[t, i]) * up[t, i]; ``gate_up`` is a tensor or ``SlicedSums`` whose rows hold the gates
+    and then the ups (gate i at i, up i at I + i) or, with ``fours``, what a product against ``rows_in_fours``
+    leaves."""
     gptr, slices, stride, rows, two_i, dtype = _branch_args(gate_up, "gated_act")
     _need(two_i % 2 == 0, "gated_act: width must be even")
     inter = two_i // 2
@@ -216,7 +234,7 @@ def gated_act(gate_up, activation: str, out: Optional[torch.Tensor] = None) -> t
     _need(out.shape == (rows, inter) and out.dtype == dtype, "gated_act: bad out")
     _need(activation in ACTIVATIONS, f"gated_act: unknown activation {activation!r}")
     _check(library().rv_gated_act(_stream(), gptr, _c_int(slices), _c_ll(stride), _ptr(out), _dt(out), _c_int(rows),
-                                  _c_int(inter), _c_int(ACTIVATIONS[activation])))
+                                  _c_int(inter), _c_int(ACTIVATIONS[activation]), _c_int(int(fours))))
     return out
 
 
@@ -560,37 +578,29 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
 
 
 SKINNY_MAX_ROWS = 64
-GATED_GEMM_MAX_ROWS = 16
 
 
-def gemm_bf16_gated(gate_up: torch.Tensor, w: torch.Tensor, activation: str, out_dtype: Optional[torch.dtype] = None,
-                    sliced_ok: bool = False):
-    """(act(gate) * up) @ w^T for a bf16 ``gate_up`` of ``[rows, 2K]`` (gates, then ups) with few rows: the
-    activation is applied while the product stages its input, which saves a kernel and a pass over memory.  None
-    when this kernel does not cover the case (the caller then applies ``gated_act`` and multiplies)."""
-    if not isinstance(gate_up, torch.Tensor) or gate_up.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+def gemm_bf16_gate_up(x: torch.Tensor, w_fours: torch.Tensor, activation: str):
+    """act(x @ gate^T) * (x @ up^T) in one kernel, for a bf16 ``x`` of at most 64 rows and ``w_fours`` =
+    ``rows_in_fours(gate, up)``: the product applies the activation where it holds the sums, which saves a kernel
+    and a pass over memory.  None when the kernel does not cover the case (rows, alignment, a shape whose product
+    is split along K): the caller then multiplies and applies ``gated_act(..., fours=True)``."""
+    if x.dtype != torch.bfloat16 or w_fours.dtype != torch.bfloat16:
         return None
-    m, two_k = gate_up.shape
-    n, k = w.shape
-    if m > GATED_GEMM_MAX_ROWS or two_k != 2 * k or k % 8 or gate_up.stride(1) != 1 or w.stride(1) != 1:
+    m, k = x.shape
+    n = w_fours.shape[0]
+    if m < 1 or m > SKINNY_MAX_ROWS or w_fours.shape[1] != k or k % 8 or n % 4 or x.stride(1) != 1 or w_fours.stride(1) != 1:
         return None
-    if (m > 1 and gate_up.stride(0) % 8) or (n > 1 and w.stride(0) % 8) or gate_up.data_ptr() % 16 or w.data_ptr() % 16:
+    if (m > 1 and x.stride(0) % 8) or (n > 1 and w_fours.stride(0) % 8) or x.data_ptr() % 16 or w_fours.data_ptr() % 16:
         return None
-    _need(gate_up.is_cuda and w.is_cuda, "gemm: arguments must live on the GPU")
-    _need(activation in ACTIVATIONS, f"gemm_bf16_gated: unknown activation {activation!r}")
+    _need(x.is_cuda and w_fours.is_cuda, "gemm: arguments must live on the GPU")
+    _need(activation in ACTIVATIONS, f"gemm_bf16_gate_up: unknown activation {activation!r}")
     lib = library()
-    out_dtype = out_dtype or gate_up.dtype
-    ldx = gate_up.stride(0) if m > 1 else two_k
-    ldw = w.stride(0) if n > 1 else k
-    slices = lib.rv_gemm_skinny_slices(_c_int(n), _c_int(k))
-    act = _c_int(ACTIVATIONS[activation])
-    if sliced_ok and slices > 1:
-        part = torch.empty((slices, m, n), dtype=torch.float32, device=w.device)
-        _check(lib.rv_gemm_skinny_gated(_stream(), _ptr(gate_up), _ptr(w), None, _c_int(_DT[out_dtype]), _ptr(part),
-                                        _c_int(m), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(n), _c_int(0), act))
-        return SlicedSums(part, out_dtype)
-    out = torch.empty((m, n), dtype=out_dtype, device=w.device)
-    part = torch.empty(slices * m * n, dtype=torch.float32, device=w.device) if slices > 1 else None
-    _check(lib.rv_gemm_skinny_gated(_stream(), _ptr(gate_up), _ptr(w), _ptr(out), _dt(out), _ptr(part), _c_int(m),
-                                    _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(n), _c_int(1), act))
+    if lib.rv_gemm_skinny_slices(_c_int(n), _c_int(k)) != 1:
+        return None
+    out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    _check(lib.rv_gemm_skinny_gate_up(_stream(), _ptr(x), _ptr(w_fours), _ptr(out), _dt(out), _c_int(m), _c_int(n),
+                                      _c_int(k), _c_ll(x.stride(0) if m > 1 else k),
+                                      _c_ll(w_fours.stride(0) if n > 1 else k), _c_ll(n // 2),
+                                      _c_int(ACTIVATIONS[activation])))
     return out

@@ -1,8 +1,10 @@
 """Dense gated feed-forward: down(act(gate(x)) * up(x)).
 
-gate and up are one product against their joined rows, gate rows first
-(v3/crates/rvllm-loader/src/gemma4_load.rs:683-685); the activation is a
-parameter (tanh-form GELU for Gemma: v3/kernels/fused_gelu_mul_f16.cu:20-27).
+gate and up are one product against their joined rows
+(v3/crates/rvllm-loader/src/gemma4_load.rs:683-685: gate rows first; here the
+rows lie in fours, two gates and then their two ups, so that the product for a
+few rows can apply the activation itself); the activation is a parameter
+(tanh-form GELU for Gemma: v3/kernels/fused_gelu_mul_f16.cu:20-27).
 """
 
 from __future__ import annotations
@@ -16,9 +18,6 @@ from .registry import FEED_FORWARDS
 from .spec import PartSpec
 
 
-FUSED_ACTIVATION_MAX_ROWS = 4
-
-
 class GatedMLP(FeedForward):
     def __init__(self, spec: PartSpec, *, hidden_size: int):
         self.hidden_size = int(hidden_size)
@@ -27,6 +26,7 @@ class GatedMLP(FeedForward):
         if self.activation not in ops.ACTIVATIONS:
             raise ValueError(f"unknown activation {self.activation!r}; known: {sorted(ops.ACTIVATIONS)}")
         self.w_gate_up = self.w_down = None
+        self.fours = False
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
         p = f"{prefix}.mlp"
@@ -40,18 +40,16 @@ class GatedMLP(FeedForward):
         p = f"{prefix}.mlp"
         gate = tensors[f"{p}.gate_proj.weight"].to(device=device, dtype=dtype)
         up = tensors[f"{p}.up_proj.weight"].to(device=device, dtype=dtype)
-        self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
+        # widths that the activation kernel cannot take in fours keep the gates before the ups
+        self.fours = self.intermediate_size % ops.FOURS_WIDTH_MULTIPLE == 0
+        self.w_gate_up = ops.rows_in_fours(gate, up) if self.fours else torch.cat([gate, up], dim=0).contiguous()
         self.w_down = tensors[f"{p}.down_proj.weight"].to(device=device, dtype=dtype).contiguous()
 
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
-        gate_up = linear(x, self.w_gate_up, sliced_ok=True)
-        # a few rows in bf16: the down product applies the activation itself while it stages its input
-        # (measured on MI355X: a gain up to 4 rows, a loss from 8 on, where every block repeats too much of it)
-        if x.shape[0] <= FUSED_ACTIVATION_MAX_ROWS:
-            fused = ops.gemm_bf16_gated(gate_up, self.w_down, self.activation, sliced_ok=True)
-            if fused is not None:
-                return fused
-        act = ops.gated_act(gate_up, self.activation)
+        # a few rows in bf16: the product applies the activation itself where it holds the sums
+        act = ops.gemm_bf16_gate_up(x, self.w_gate_up, self.activation) if self.fours and x.is_cuda else None
+        if act is None:
+            act = ops.gated_act(linear(x, self.w_gate_up, sliced_ok=True), self.activation, fours=self.fours)
         return linear(act, self.w_down, sliced_ok=True)
 
 

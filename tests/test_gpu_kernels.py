@@ -153,29 +153,46 @@ def test_gemm_skinny(m, n, k, out_dtype):
 
 
 @pytest.mark.parametrize("activation", ["gelu_pytorch_tanh", "silu"])
-@pytest.mark.parametrize("m,n,k", [(1, 40, 64), (8, 96, 1416), (16, 2560, 10240), (5, 33, 520)])
-def test_gemm_with_the_gated_activation_in_its_staging(m, n, k, activation):
-    """(act(gate) * up) @ W^T in one kernel: against 64-bit arithmetic, and bit for bit against the
-    activation kernel followed by the product (both round the activation to bf16 the same way)."""
+@pytest.mark.parametrize("m,inter,k", [(1, 40, 64), (8, 96, 128), (64, 10240, 2560), (5, 520, 96), (17, 8, 8)])
+def test_gate_and_up_product_with_the_activation_in_it(m, inter, k, activation):
+    """act(x gate^T) * (x up^T) in one kernel over the rows in fours: against 64-bit arithmetic, and bit for bit
+    against the product followed by the activation kernel, with the rows in fours and with the gates before the
+    ups (all round the sums to bf16 before the activation)."""
     g = torch.Generator().manual_seed(22)
-    gate_up = (torch.randn(m, 2 * k, generator=g) * 1.5).bfloat16()
-    gate_up[0, :4] = torch.tensor([-30.0, 30.0, 0.0, -0.0]).bfloat16()  # the ends of the activation's range
-    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
-    fused = ops.gemm_bf16_gated(dev(gate_up), dev(w), activation, out_dtype=torch.float32)
-    assert fused is not None and fused.shape == (m, n)
-    gd, ud = gate_up[:, :k].double(), gate_up[:, k:].double()
-    act = F.gelu(gd, approximate="tanh") if activation != "silu" else F.silu(gd)
-    want = (act * ud).bfloat16().double() @ w.double().T
-    scale = want.abs().max().item()
-    assert (fused.cpu().double() - want).abs().max().item() <= 2e-3 * scale * max(1.0, math.sqrt(k) / 16)
-    two_step = ops.gemm_bf16(ops.gated_act(dev(gate_up), activation), dev(w), out_dtype=torch.float32)
-    assert torch.equal(fused, two_step)
-    # unreduced slices, as the norm after it takes them
-    sums = ops.gemm_bf16_gated(dev(gate_up), dev(w), activation, sliced_ok=True)
-    assert torch.allclose(ops.as_tensor(sums).float(), fused, atol=2e-2 * scale, rtol=0)
-    # more rows than it covers, or another type: left to the two kernels
-    assert ops.gemm_bf16_gated(dev(torch.zeros(17, 2 * k).bfloat16()), dev(w), activation) is None
-    assert ops.gemm_bf16_gated(dev(gate_up.float()), dev(w.float()), activation) is None
+    x = (torch.randn(m, k, generator=g) * 1.5).bfloat16()
+    gate = (torch.randn(inter, k, generator=g) * 0.08).bfloat16()
+    up = (torch.randn(inter, k, generator=g) * 0.08).bfloat16()
+    gate[:2], up[:2] = gate[:2] * 40, up[:2] * 0  # far out on the activation, and exact zeros
+    fours = ops.rows_in_fours(gate, up)
+    assert fours.shape == (2 * inter, k) and torch.equal(fours[0], gate[0]) and torch.equal(fours[1], gate[1])
+    assert torch.equal(fours[2], up[0]) and torch.equal(fours[3], up[1]) and torch.equal(fours[4], gate[2])
+    fused = ops.gemm_bf16_gate_up(dev(x), dev(fours), activation)
+    assert fused is not None and fused.shape == (m, inter) and fused.dtype == torch.bfloat16
+    gd, ud = (x.double() @ gate.double().T).bfloat16().double(), (x.double() @ up.double().T).bfloat16().double()
+    want = (F.gelu(gd, approximate="tanh") if activation != "silu" else F.silu(gd)) * ud
+    assert torch.allclose(fused.cpu().float(), want.float(), **tol(torch.bfloat16))
+    in_fours = ops.gated_act(ops.gemm_bf16(dev(x), dev(fours)), activation, fours=True)
+    halves = ops.gated_act(ops.gemm_bf16(dev(x), dev(torch.cat([gate, up]))), activation)
+    assert torch.equal(fused, in_fours) and torch.equal(fused, halves)
+    # another type, more rows than it covers, or a shape whose product is split along K: left to the two kernels
+    assert ops.gemm_bf16_gate_up(dev(x.float()), dev(fours.float()), activation) is None
+    assert ops.gemm_bf16_gate_up(dev(torch.zeros(65, k).bfloat16()), dev(fours), activation) is None
+    assert ops.gemm_bf16_gate_up(dev(torch.zeros(8, 1416).bfloat16()), dev(torch.zeros(192, 1416).bfloat16()), activation) is None
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gated_act_over_rows_in_fours(dtype):
+    """Whole values and unreduced slices; a width that the kernel cannot take in fours is refused."""
+    g = torch.Generator().manual_seed(23)
+    gate, up = torch.randn(5, 48, generator=g).to(dtype), torch.randn(5, 48, generator=g).to(dtype)
+    gu = ops.rows_in_fours(gate.T.contiguous(), up.T.contiguous()).T.contiguous()  # the columns in fours
+    want = (F.silu(gate.double()) * up.double()).float()
+    assert torch.allclose(ops.gated_act(dev(gu), "silu", fours=True).cpu().float(), want, **tol(dtype))
+    parts = torch.stack([gu.float() * 0.25, gu.float() * 0.75])
+    sums = ops.SlicedSums(dev(parts), dtype)
+    assert torch.allclose(ops.gated_act(sums, "silu", fours=True).cpu().float(), want, **tol(dtype))
+    with pytest.raises(ops.KernelError, match="multiple of"):
+        ops.gated_act(dev(torch.zeros(2, 2 * 42, dtype=dtype)), "silu", fours=True)
 
 
 def test_gemm_skinny_reads_strided_rows_and_refuses_what_it_cannot():
