@@ -56,3 +56,24 @@ def test_cuttings_at_the_4b_layer_sizes(model, dtype, mode):
         tt.compare(got[f"{prefix}-{name}"], ref, dtype, f"4B layer sizes, {dtype}, {mode}, {name}")
     assert all(free == g.pool.num_pages for free, g in zip(runner.cache.free_pages().values(),
                                                            runner.cache.groups.values()))
+
+
+@pytest.mark.parametrize("mode", ["portions", "mixed"])
+def test_a_cache_that_held_nan_before_at_the_4b_layer_sizes(model, mode):
+    """Pages come with what their last holder left, which need not be finite:
+    every slot of the cache is NaN before the first step, and no logit may show
+    it (the slots beyond a request's newest token are left out, not multiplied
+    by zero)."""
+    folder, cfg, seqs, refs = model
+    steps = MODES[mode](seqs)
+    most = tt.required_tokens(steps)
+    runner = ModelRunner.from_model_dir(folder, EngineConfig(
+        dtype="bfloat16", page_size=16, max_model_len=max(LENGTHS) + 20, max_num_seqs=2, max_num_batched_tokens=most,
+        max_prefill_chunk=most, max_cache_tokens=most))
+    for view in runner.storage.views:
+        view.k_pages.fill_(float("nan"))
+        view.v_pages.fill_(float("nan"))
+    got = tt.collect(steps, tt.run_in_process(runner, steps), cfg["vocab"])
+    prefix = steps[0]["entries"][0]["id"].split("-")[0]
+    for name, ref in refs.items():
+        tt.compare(got[f"{prefix}-{name}"], ref, "bfloat16", f"4B layer sizes, NaN pages, {mode}, {name}")

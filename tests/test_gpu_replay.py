@@ -82,6 +82,29 @@ def test_cuttings_agree_bit_for_bit_in_32_bit(model_dirs, references, name):
             assert np.array_equal(results[mode][rid], results["whole"][rid]), f"{name} {mode} {rid}"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+@pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
+def test_what_a_page_held_before_reaches_no_logit(model_dirs, references, name, dtype, mode):
+    """A page comes to a request with whatever its last holder left in it, and
+    that need not be finite.  Here every slot of the cache holds NaN before the
+    first step: a kernel that multiplies a slot beyond the request's newest
+    token by a probability of zero, instead of leaving it out, shows it."""
+    seqs, refs = references[name]
+    vocab = next(iter(refs.values())).shape[1]
+    steps = MODES[mode](seqs)
+    runner = make_runner(model_dirs[name], dtype, max_tokens=tt.required_tokens(steps))
+    poisoned = 0
+    for view in runner.storage.views:
+        if view is not None and hasattr(view, "k_pages"):
+            view.k_pages.fill_(float("nan"))
+            view.v_pages.fill_(float("nan"))
+            poisoned += 1
+    assert poisoned > 0
+    outputs = tt.run_in_process(runner, steps)
+    check(steps, outputs, refs, vocab, dtype, steps[0]["entries"][0]["id"].split("-")[0], f"NaN pages {name} {dtype} {mode}")
+
+
 @pytest.mark.parametrize("page_size", [32, 64])
 def test_other_page_sizes(model_dirs, references, page_size):
     seqs, refs = references["B"]
