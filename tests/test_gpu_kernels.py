@@ -528,6 +528,22 @@ def test_paged_attention_mfma_every_split(splits, window):
     assert torch.allclose(got.float(), want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("nq,nkv,hd", [(6, 1, 48), (3, 3, 80), (8, 4, 256), (16, 1, 32), (4, 2, 128)])
+@pytest.mark.parametrize("splits", [(19, 64), (38, 32)])
+def test_paged_attention_mfma_merges_many_splits(nq, nkv, hd, splits):
+    """Many splits of the keys, merged afterwards: more splits than the merge
+    loads at a time, tiles of one, two and three tokens, head counts that
+    leave columns of a tile empty, head sizes that are no power of two; and
+    again right away, into a workspace that holds the last call's parts."""
+    portions = [(1199, 1), (1100, 2), (0, 3), (700, 1), (1213, 1)]
+    for window in (None, 300):
+        case = Case(portions, nq, nkv, hd, 16, torch.bfloat16, 17, window)
+        want = case.reference(hd ** -0.5).float()
+        for again in range(3):
+            got = case.run("mfma", hd ** -0.5, splits=splits, prefill_kernel=False).float()
+            assert torch.allclose(got, want, **tol(torch.bfloat16)), (window, again)
+
+
 def test_paged_attention_mfma_long_decode_batch():
     """Decode shapes: many requests with one token each at long, different contexts."""
     portions = [(4000 + 37 * i, 1) for i in range(9)]
