@@ -187,13 +187,14 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, const int* __restrict__ 
   const int in_row = row_index ? row_index[blockIdx.x] : (int)blockIdx.x;
   const T* xr = x + (size_t)in_row * width;
   T* yr = y + (size_t)blockIdx.x * width;
-  float val[E][V];
+  float val[E][V], g[E][V];  // the weights are asked for with the row, not after the sum's barrier
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < E; ++e) {
     const int i = (e * blockDim.x + threadIdx.x) * V;
     if (i < width) {
       row_load<T, V>(xr + i, val[e]);
+      row_load_w<V>(w, w_f32, i, g[e]);
 #pragma unroll
       for (int v = 0; v < V; ++v) ss += val[e][v] * val[e][v];
     }
@@ -204,10 +205,8 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, const int* __restrict__ 
   for (int e = 0; e < E; ++e) {
     const int i = (e * blockDim.x + threadIdx.x) * V;
     if (i < width) {
-      float g[V];
-      row_load_w<V>(w, w_f32, i, g);
 #pragma unroll
-      for (int v = 0; v < V; ++v) val[e][v] = val[e][v] * inv * (offset + g[v]);
+      for (int v = 0; v < V; ++v) val[e][v] = val[e][v] * inv * (offset + g[e][v]);
       row_store<T, V>(yr + i, val[e]);
     }
   }
@@ -267,13 +266,18 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ branch, int slices, 
   __shared__ float scratch[16];
   const size_t row0 = (size_t)blockIdx.x * width;
   T* rr = residual + row0;
-  float val[E][V];
+  // Everything the row needs is asked for at once, before the first sum: a load behind a barrier would only
+  // start after it, and at a few rows a step the kernel is as long as its chain of round trips to memory.
+  float val[E][V], res[E][V], g_post[E][V], g_next[E][V];
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < E; ++e) {
     const int i = (e * blockDim.x + threadIdx.x) * V;
     if (i < width) {
       row_load_branch<T, V>(branch, slices, slice_stride, row0 + i, val[e]);
+      row_load<T, V>(rr + i, res[e]);
+      row_load_w<V>(w_post, w_post_f32, i, g_post[e]);
+      if (next != nullptr) row_load_w<V>(w_next, w_next_f32, i, g_next[e]);
 #pragma unroll
       for (int v = 0; v < V; ++v) ss += val[e][v] * val[e][v];
     }
@@ -285,13 +289,10 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ branch, int slices, 
   for (int e = 0; e < E; ++e) {
     const int i = (e * blockDim.x + threadIdx.x) * V;
     if (i < width) {
-      float g[V], r[V];
-      row_load_w<V>(w_post, w_post_f32, i, g);
-      row_load<T, V>(rr + i, r);
 #pragma unroll
       for (int v = 0; v < V; ++v) {
         // the residual as it reads back after the store
-        val[e][v] = rv_round_to<T>(r[v] + val[e][v] * inv * (offset + g[v]));
+        val[e][v] = rv_round_to<T>(res[e][v] + val[e][v] * inv * (offset + g_post[e][v]));
         ss2 += val[e][v] * val[e][v];
       }
       row_store<T, V>(rr + i, val[e]);
@@ -305,10 +306,8 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ branch, int slices, 
   for (int e = 0; e < E; ++e) {
     const int i = (e * blockDim.x + threadIdx.x) * V;
     if (i < width) {
-      float g[V];
-      row_load_w<V>(w_next, w_next_f32, i, g);
 #pragma unroll
-      for (int v = 0; v < V; ++v) val[e][v] = val[e][v] * inv2 * (offset_next + g[v]);
+      for (int v = 0; v < V; ++v) val[e][v] = val[e][v] * inv2 * (offset_next + g_next[e][v]);
       row_store<T, V>(nr + i, val[e]);
     }
   }

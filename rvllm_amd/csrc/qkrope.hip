@@ -329,6 +329,16 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
   const int i0 = first_half ? d0 : d0 - hd / 2;  // index of the lane's pairs
   const int rot_half = rot / 2;
 
+  // Everything is asked for up front and from places that are always there, so that no read waits behind another
+  // or behind a branch: at a few tokens a step this kernel is as long as its chain of round trips to memory.
+  // First the token's place in the cache, which is two reads one after the other.
+  const bool to_cache = !is_q && write_kv != 0;
+  int pos = 0, req = 0;
+  if (write_kv != 0) {  // the same for the whole launch
+    pos = positions[t];
+    req = token_req[t];
+  }
+
   // the head's values: stored as T, or the sums of the product's K slices in their order
   float x[4] = {0.f, 0.f, 0.f, 0.f};
   if (slices == 0) {
@@ -357,25 +367,25 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
   const bool normed = w != nullptr && (is_q || is_k);
   const bool rotates = (is_q || is_k) && active && i0 < rot_half;
   float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f}, g[4] = {0.f, 0.f, 0.f, 0.f};
-  if (rotates) {
-    QkrVec<float>::load(rope_cos + (size_t)t * rot_half + i0, c);
-    QkrVec<float>::load(rope_sin + (size_t)t * rot_half + i0, sn);
+  if (rot_half > 0) {  // the same for the whole launch; a lane that does not rotate reads the first pairs and drops them
+    const int i_safe = rotates ? i0 : 0;
+    QkrVec<float>::load(rope_cos + (size_t)t * rot_half + i_safe, c);
+    QkrVec<float>::load(rope_sin + (size_t)t * rot_half + i_safe, sn);
   }
-  if (normed) {
+  if (w != nullptr) {  // the same for the whole wave
 #pragma unroll
     for (int j = 0; j < 4; ++j) g[j] = rv_load_w(w, w_f32, d0 + j);
   }
+  const int logical = write_kv != 0 ? pos / page_size : 0;  // without a cache there is no page size either
+  const bool in_table = to_cache && logical < table_width;
+  int page = -1;
+  if (write_kv != 0) page = block_table[(size_t)req * table_width + (in_table ? logical : 0)];
+  if (!in_table) page = -1;
 
   T* dst = nullptr;
   if (is_q) {
     dst = q_out + ((size_t)t * nq + head) * hd;
   } else {
-    if (!write_kv) return;
-    const int pos = positions[t];
-    const int req = token_req[t];
-    const int logical = pos / page_size;
-    if (logical >= table_width) return;
-    const int page = block_table[(size_t)req * table_width + logical];
     if (page < 0 || page >= num_pages) return;
     const int slot = pos % page_size;
     if (is_k) {
