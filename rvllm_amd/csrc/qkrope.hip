@@ -297,7 +297,10 @@ struct QkrVec<bf16_t> {
   }
 };
 
-template <typename T>
+// A wave takes HPW heads of one token, one after the other with all their reads asked for at once: the token's
+// place in the cache and its cosines and sines, four times a head's bytes, are then fetched once for all of them.
+// (One head a wave, a prompt portion is tens of thousands of waves that each fetch those again.)
+template <typename T, int HPW>
 __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, int slices, long long slice_stride,
                                                  T* __restrict__ q_out, const void* __restrict__ q_w,
                                                  const void* __restrict__ k_w, int w_f32, float eps, float offset,
@@ -305,121 +308,132 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
                                                  int rot, const int* __restrict__ positions,
                                                  const int* __restrict__ token_req, const int* __restrict__ block_table,
                                                  int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                                 int page_size, int num_pages, int nq, int nkv, int hd, int write_kv, ValuePages V) {
+                                                 int page_size, int num_pages, int nq, int nkv, int hd, int write_kv,
+                                                 ValuePages V) {
   const int wave = threadIdx.x / RV_WAVE;
   const int lane = threadIdx.x & (RV_WAVE - 1);
-  const int head_rows = ((write_kv == 1 ? nq + 2 * nkv : nq + nkv) + 3) / 4;
+  // the heads that waves take: queries; keys and, token by token, values if they go to the cache
+  const int heads = write_kv == 0 ? nq : (write_kv == 1 ? nq + 2 * nkv : nq + nkv);
+  const int head_rows = (heads + 4 * HPW - 1) / (4 * HPW);
   if ((int)blockIdx.y >= head_rows) {  // the rows of the grid beyond the heads write values a page at a time
     v_write_page<T>((long long)(blockIdx.y - head_rows) * gridDim.x + blockIdx.x, V, (const T*)qkv, v_pages, block_table,
                     table_width, page_size, num_pages, nq, nkv, hd);
     return;
   }
   const int t = blockIdx.x;
-  const int head = blockIdx.y * 4 + wave;
+  const int head0 = (blockIdx.y * 4 + wave) * HPW;
   const int total_heads = nq + 2 * nkv;
-  if (head >= total_heads) return;  // whole wave leaves together; there is no block barrier below
+  if (head0 >= heads) return;  // whole wave leaves together; there is no block barrier below
 
-  const size_t src = (size_t)t * total_heads * hd + (size_t)head * hd;  // first element of this head in qkv
-  const bool is_q = head < nq;
-  const bool is_k = !is_q && head < nq + nkv;
   const int half_lanes = hd / 8;          // lanes that hold one half of the head
   const bool active = lane < 2 * half_lanes;
   const int d0 = active ? lane * 4 : 0;   // a lane without dimensions reads a valid place and drops it
   const bool first_half = lane < half_lanes;
   const int i0 = first_half ? d0 : d0 - hd / 2;  // index of the lane's pairs
   const int rot_half = rot / 2;
+  const bool lane_rotates = active && i0 < rot_half;
 
   // Everything is asked for up front and from places that are always there, so that no read waits behind another
   // or behind a branch: at a few tokens a step this kernel is as long as its chain of round trips to memory.
   // First the token's place in the cache, which is two reads one after the other.
-  const bool to_cache = !is_q && write_kv != 0;
   int pos = 0, req = 0;
   if (write_kv != 0) {  // the same for the whole launch
     pos = positions[t];
     req = token_req[t];
   }
-
-  // the head's values: stored as T, or the sums of the product's K slices in their order
-  float x[4] = {0.f, 0.f, 0.f, 0.f};
-  if (slices == 0) {
-    QkrVec<T>::load((const T*)qkv + src + d0, x);
-  } else {
-    const float* p = (const float*)qkv + src + d0;
-    int s = 0;
-    for (; s + 4 <= slices; s += 4) {  // four reads in flight
-      const float4 a = *(const float4*)(p + (size_t)s * slice_stride);
-      const float4 b = *(const float4*)(p + (size_t)(s + 1) * slice_stride);
-      const float4 c = *(const float4*)(p + (size_t)(s + 2) * slice_stride);
-      const float4 d = *(const float4*)(p + (size_t)(s + 3) * slice_stride);
-      x[0] = (((x[0] + a.x) + b.x) + c.x) + d.x;
-      x[1] = (((x[1] + a.y) + b.y) + c.y) + d.y;
-      x[2] = (((x[2] + a.z) + b.z) + c.z) + d.z;
-      x[3] = (((x[3] + a.w) + b.w) + c.w) + d.w;
+  // the heads' values: stored as T, or the sums of the product's K slices in their order; a head beyond the last
+  // repeats the last one and stores nothing
+  float x[HPW][4];
+#pragma unroll
+  for (int j = 0; j < HPW; ++j) {
+    const int head = head0 + j < heads ? head0 + j : heads - 1;
+    const size_t src = (size_t)t * total_heads * hd + (size_t)head * hd;  // first element of this head in qkv
+    x[j][0] = x[j][1] = x[j][2] = x[j][3] = 0.f;
+    if (slices == 0) {
+      QkrVec<T>::load((const T*)qkv + src + d0, x[j]);
+    } else {
+      const float* p = (const float*)qkv + src + d0;
+      int s = 0;
+      for (; s + 4 <= slices; s += 4) {  // four reads in flight
+        const float4 a = *(const float4*)(p + (size_t)s * slice_stride);
+        const float4 b = *(const float4*)(p + (size_t)(s + 1) * slice_stride);
+        const float4 c = *(const float4*)(p + (size_t)(s + 2) * slice_stride);
+        const float4 d = *(const float4*)(p + (size_t)(s + 3) * slice_stride);
+        x[j][0] = (((x[j][0] + a.x) + b.x) + c.x) + d.x;
+        x[j][1] = (((x[j][1] + a.y) + b.y) + c.y) + d.y;
+        x[j][2] = (((x[j][2] + a.z) + b.z) + c.z) + d.z;
+        x[j][3] = (((x[j][3] + a.w) + b.w) + c.w) + d.w;
+      }
+      for (; s < slices; ++s) {
+        const float4 a = *(const float4*)(p + (size_t)s * slice_stride);
+        x[j][0] += a.x, x[j][1] += a.y, x[j][2] += a.z, x[j][3] += a.w;
+      }
     }
-    for (; s < slices; ++s) {
-      const float4 a = *(const float4*)(p + (size_t)s * slice_stride);
-      x[0] += a.x, x[1] += a.y, x[2] += a.z, x[3] += a.w;
-    }
+    if (!active) x[j][0] = x[j][1] = x[j][2] = x[j][3] = 0.f;
   }
-  if (!active) x[0] = x[1] = x[2] = x[3] = 0.f;
-
-  const void* w = is_q ? q_w : k_w;
-  const bool normed = w != nullptr && (is_q || is_k);
-  const bool rotates = (is_q || is_k) && active && i0 < rot_half;
-  float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f}, g[4] = {0.f, 0.f, 0.f, 0.f};
+  float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
   if (rot_half > 0) {  // the same for the whole launch; a lane that does not rotate reads the first pairs and drops them
-    const int i_safe = rotates ? i0 : 0;
+    const int i_safe = lane_rotates ? i0 : 0;
     QkrVec<float>::load(rope_cos + (size_t)t * rot_half + i_safe, c);
     QkrVec<float>::load(rope_sin + (size_t)t * rot_half + i_safe, sn);
   }
-  if (w != nullptr) {  // the same for the whole wave
+  float g_q[4] = {0.f, 0.f, 0.f, 0.f}, g_k[4] = {0.f, 0.f, 0.f, 0.f};
+  if (q_w != nullptr) {  // the same for the whole launch; the weights of queries and keys come together
 #pragma unroll
-    for (int j = 0; j < 4; ++j) g[j] = rv_load_w(w, w_f32, d0 + j);
+    for (int i = 0; i < 4; ++i) {
+      g_q[i] = rv_load_w(q_w, w_f32, d0 + i);
+      g_k[i] = rv_load_w(k_w, w_f32, d0 + i);
+    }
   }
   const int logical = write_kv != 0 ? pos / page_size : 0;  // without a cache there is no page size either
-  const bool in_table = to_cache && logical < table_width;
+  const bool in_table = write_kv != 0 && logical < table_width;
   int page = -1;
   if (write_kv != 0) page = block_table[(size_t)req * table_width + (in_table ? logical : 0)];
-  if (!in_table) page = -1;
+  if (!in_table || page >= num_pages) page = -1;
+  const int slot = write_kv != 0 ? pos % page_size : 0;
 
-  T* dst = nullptr;
-  if (is_q) {
-    dst = q_out + ((size_t)t * nq + head) * hd;
-  } else {
-    if (page < 0 || page >= num_pages) return;
-    const int slot = pos % page_size;
-    if (is_k) {
-      dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
+#pragma unroll
+  for (int j = 0; j < HPW; ++j) {
+    const int head = head0 + j;
+    if (head >= heads) break;  // the same for the whole wave, as all that follows
+    const bool is_q = head < nq;
+    const bool is_k = !is_q && head < nq + nkv;
+    T* dst = nullptr;
+    if (is_q) {
+      dst = q_out + ((size_t)t * nq + head) * hd;
     } else {
-      if (write_kv == 2) return;  // values are written a page at a time by other blocks of this launch
-      // values are stored as projected, transposed inside the page
-      T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
-      if (active) {
+      if (page < 0) continue;
+      if (is_k) {
+        dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
+      } else {
+        // values are stored as projected, transposed inside the page
+        T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
+        if (active) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) col[(size_t)(d0 + j) * page_size] = rv_from_float<T>(x[j]);
+          for (int i = 0; i < 4; ++i) col[(size_t)(d0 + i) * page_size] = rv_from_float<T>(x[j][i]);
+        }
+        continue;
       }
-      return;
     }
-  }
-
-  if (normed) {
-    float ss = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
-    ss = rv_wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+    if (q_w != nullptr) {
+      float ss = x[j][0] * x[j][0] + x[j][1] * x[j][1] + x[j][2] * x[j][2] + x[j][3] * x[j][3];
+      ss = rv_wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) x[j] = x[j] * inv * (offset + g[j]);
-  }
-  if (rot_half > 0) {
-    // the other half of each pair sits hd/8 lanes away; every lane takes part in the exchange
-    const int partner = first_half ? lane + half_lanes : lane - half_lanes;
-    const int from = active ? partner : lane;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float other = __shfl(x[j], from, RV_WAVE);
-      if (rotates) x[j] = first_half ? x[j] * c[j] - other * sn[j] : x[j] * c[j] + other * sn[j];
+      for (int i = 0; i < 4; ++i) x[j][i] = x[j][i] * inv * (offset + (is_q ? g_q[i] : g_k[i]));
     }
+    if (rot_half > 0) {
+      // the other half of each pair sits hd/8 lanes away; every lane takes part in the exchange
+      const int partner = first_half ? lane + half_lanes : lane - half_lanes;
+      const int from = active ? partner : lane;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float other = __shfl(x[j][i], from, RV_WAVE);
+        if (lane_rotates) x[j][i] = first_half ? x[j][i] * c[i] - other * sn[i] : x[j][i] * c[i] + other * sn[i];
+      }
+    }
+    if (active) QkrVec<T>::store(dst + d0, x[j]);
   }
-  if (active) QkrVec<T>::store(dst + d0, x);
 }
 
 // `slices` 0: qkv holds T values [tokens, (nq + 2 nkv) * hd]; otherwise 32-bit
@@ -447,7 +461,12 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
   // not partial sums)
   RV_CHECK(write_kv >= 0 && write_kv <= 2, "qk_norm_rope: write_kv is 0, 1 or 2");
   ValuePages V = {q_start, chunk_start, num_requests, 0};
-  int rows = rv_div_up(write_kv == 1 ? nq + 2 * nkv : nq + nkv, 4);
+  const bool vec = hd % 8 == 0 && hd <= 4 * RV_WAVE && rot % 8 == 0;  // four dimensions a lane
+  // the heads that waves take: queries; keys and, token by token, values if they go to the cache
+  const int heads = write_kv == 0 ? nq : (write_kv == 1 ? nq + 2 * nkv : nq + nkv);
+  // a prompt portion's waves take four heads each; a few tokens' take one, spread over the machine
+  const int hpw = vec && num_tokens >= 256 ? 4 : 1;
+  int rows = rv_div_up(vec ? heads : (write_kv == 1 ? nq + 2 * nkv : nq + nkv), 4 * hpw);
   if (write_kv == 2) {
     RV_CHECK(slices == 0 && q_start && chunk_start && num_requests >= 1 && max_portion >= 1,
              "qk_norm_rope: values by pages need the step's portions and a projection that is already added up");
@@ -457,22 +476,22 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
     RV_CHECK(rows <= 65535, "qk_norm_rope: too many pages of values for one launch");
   }
   dim3 grid(num_tokens, rows), block(4 * RV_WAVE);
-  if (hd % 8 == 0 && hd <= 4 * RV_WAVE && rot % 8 == 0) {  // four dimensions a lane
-    if (dtype == RV_F32)
-      qk_norm_rope_kv_write_vec_kernel<float><<<grid, block, 0, stream>>>(
-          qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions,
-          token_req, block_table, table_width, (float*)k_pages, (float*)v_pages, page_size, num_pages, nq, nkv, hd,
-          write_kv, V);
-    else if (dtype == RV_BF16)
-      qk_norm_rope_kv_write_vec_kernel<bf16_t><<<grid, block, 0, stream>>>(
-          qkv, slices, slice_stride, (bf16_t*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions,
-          token_req, block_table, table_width, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, num_pages, nq, nkv, hd,
-          write_kv, V);
-    else
+#define QKR_VEC_LAUNCH(TT, HPW)                                                                                        \
+  qk_norm_rope_kv_write_vec_kernel<TT, HPW><<<grid, block, 0, stream>>>(                                               \
+      qkv, slices, slice_stride, (TT*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions,         \
+      token_req, block_table, table_width, (TT*)k_pages, (TT*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv, V)
+  if (vec) {
+    if (dtype == RV_F32) {
+      if (hpw == 4) QKR_VEC_LAUNCH(float, 4); else QKR_VEC_LAUNCH(float, 1);
+    } else if (dtype == RV_BF16) {
+      if (hpw == 4) QKR_VEC_LAUNCH(bf16_t, 4); else QKR_VEC_LAUNCH(bf16_t, 1);
+    } else {
       return rv_fail("qk_norm_rope: unsupported dtype %d", dtype);
+    }
     RV_LAUNCH_CHECK("qk_norm_rope_kv_write");
     return 0;
   }
+#undef QKR_VEC_LAUNCH
   if (dtype == RV_F32)
     qk_norm_rope_kv_write_kernel<float><<<grid, block, 0, stream>>>(
         qkv, slices, slice_stride, (float*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions, token_req,

@@ -235,8 +235,8 @@ def from_cache(kp, vp):
 @pytest.mark.parametrize("nq,nkv,hd,rot", [(4, 2, 16, 16), (6, 3, 48, 48), (5, 1, 80, 40), (8, 4, 256, 256), (3, 3, 128, 0),
                                           (2, 1, 36, 12), (2, 2, 512, 512)])  # the last two: the kernel for odd sizes
 @pytest.mark.parametrize("page_size", [16, 64])
-def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size):
-    T = 37
+@pytest.mark.parametrize("T", [37, 301])  # a few tokens: one a wave; a prompt portion: four a wave, the last wave not full
+def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size, T):
     g, k_pages, v_pages, table = paged_setup(T + 100, nkv, hd, page_size, dtype, 7)
     qkv = torch.randn(T, (nq + 2 * nkv) * hd, generator=g).to(dtype)
     qw = (torch.randn(hd, generator=g) * 0.1).to(dtype)
@@ -273,11 +273,12 @@ def test_qk_norm_rope_kv_write(dtype, nq, nkv, hd, rot, page_size):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("page_size", [16, 32])
-def test_values_written_a_page_at_a_time(dtype, page_size):
+@pytest.mark.parametrize("longest", [70, 333])  # the step's tokens one a wave, and four a wave
+def test_values_written_a_page_at_a_time(dtype, page_size, longest):
     """Portions that begin and end inside pages, cover whole pages, and single tokens: the values reach the same
     places as when every token writes its own, and nothing else is touched."""
     nq, nkv, hd = 4, 2, 48
-    portions = [(5, 70), (64, 32), (0, 1), (31, 2), (100, 16)]  # (first position, tokens)
+    portions = [(5, longest), (64, 32), (0, 1), (31, 2), (100, 16)]  # (first position, tokens)
     case = Case(portions, nq, nkv, hd, page_size, dtype, 17)
     T = case.q.shape[0]
     g = torch.Generator().manual_seed(18)
