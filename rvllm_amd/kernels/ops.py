@@ -427,6 +427,40 @@ def plan_attention_splits(num_requests: int, max_portion: int, max_context: int,
     return tiles, splits, split_len
 
 
+# The kernel that gives a tile's key splits to the eight waves of one block and merges them there, with no second
+# kernel: worth it while a wave walks few blocks of keys (a window, a short context), and possible while the
+# tile's columns fit the block's LDS.
+_ATTN_IN_BLOCK_WAVES = 8
+_ATTN_IN_BLOCK_LDS = 64 * 1024
+_ATTN_IN_BLOCK_MAX_KEY_BLOCKS = 6
+_ATTN_IN_BLOCK_MIN_TILES = 256
+
+
+def plan_attention_in_block(max_portion: int, max_context: int, group: int, window: Optional[int],
+                            head_dim: int, num_tiles: Optional[int] = None) -> Optional[tuple[int, int]]:
+    """(keys per split, columns of a tile kept in LDS) if the decode kernel is
+    to merge a tile's splits inside its block, else None.  With ``num_tiles``
+    (requests x tiles x key/value heads) the answer is also None while the
+    tiles are too few to fill the machine eight waves each: then the keys
+    are better split further, over more waves than a block has."""
+    if num_tiles is not None and num_tiles < _ATTN_IN_BLOCK_MIN_TILES:
+        return None
+    group_pad = 1
+    while group_pad < group:
+        group_pad *= 2
+    tokens_per_tile = 16 // group_pad
+    cols = min(max_portion, tokens_per_tile) * group
+    if _ATTN_IN_BLOCK_WAVES * cols * (head_dim + 2) * 4 > _ATTN_IN_BLOCK_LDS:
+        return None
+    span = max_context
+    if window:
+        span = min(span, window - 1 + 31 + tokens_per_tile)
+    per = -(-(-(-span // 32)) // _ATTN_IN_BLOCK_WAVES)  # blocks of 32 keys a wave
+    if per > _ATTN_IN_BLOCK_MAX_KEY_BLOCKS:
+        return None
+    return per * 32, cols
+
+
 # Portions of at least this many tokens go to the kernel whose blocks share key
 # tiles through LDS; shorter ones (decoded tokens above all) to the kernel that
 # splits a request's keys over many waves.
@@ -435,10 +469,12 @@ PREFILL_MIN_PORTION = 16
 
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                          step, out: torch.Tensor, num_q_heads: int, scale: float, window: Optional[int],
-                         splits: Optional[tuple[int, int]] = None, prefill_kernel: Optional[bool] = None) -> torch.Tensor:
+                         splits: Optional[tuple[int, int]] = None, prefill_kernel: Optional[bool] = None,
+                         in_block: Optional[bool] = None) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``splits`` = (number, keys per
-    split) overrides the plan and ``prefill_kernel`` the choice of kernel
-    (tests use them to force every path)."""
+    split) overrides the plan, ``prefill_kernel`` the choice of kernel and
+    ``in_block`` whether a tile's splits are merged inside one block (tests
+    use them to force every path)."""
     _gpu(q, k_pages, v_pages, block_table, out)
     _i32(block_table)
     n = q.shape[0]
@@ -486,13 +522,22 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     if shortest_rest > 0:
         tiles, num_splits, split_len = plan_attention_splits(step.num_requests, shortest_rest, step.max_context, nkv,
                                                              group, window, hd)
-        if splits is not None:
+        block_cols = 0
+        merged = None
+        if in_block is not False:
+            merged = plan_attention_in_block(shortest_rest, step.max_context, group, window, hd,
+                                             None if in_block else step.num_requests * tiles * nkv)
+        if in_block:
+            _need(merged is not None, "attention: these keys or columns are too many to merge inside a block")
+        if merged is not None and (splits is None or in_block):
+            num_splits, (split_len, block_cols) = _ATTN_IN_BLOCK_WAVES, merged
+        elif splits is not None:
             num_splits, split_len = splits
             need = -(-step.max_context // 32) * 32
             _need(window is not None or num_splits * split_len >= need,
                   "attention: the splits do not cover the context")
         part_o = part_ml = None
-        if num_splits > 1:
+        if num_splits > 1 and block_cols == 0:
             units = step.num_requests * tiles * nkv * num_splits
             part_o = torch.empty(units * 16 * hd, dtype=torch.float32, device=q.device)
             part_ml = torch.empty(units * 32, dtype=torch.float32, device=q.device)
@@ -502,7 +547,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                      _ptr(out), _ptr(part_o), _ptr(part_ml), _c_int(n), _c_int(step.num_requests), _c_int(tiles),
                      _c_int(num_q_heads), _c_int(nkv), _c_int(hd), _c_int(page_size), _c_int(num_pages),
                      _c_int(window or 0), _c_int(num_splits), _c_int(split_len),
-                     _c_int(portion_min - 1 if use_prefill else 0), _c_float(scale)))
+                     _c_int(portion_min - 1 if use_prefill else 0), _c_int(block_cols), _c_float(scale)))
     return out
 
 

@@ -545,6 +545,46 @@ def test_paged_attention_mfma_merges_many_splits(nq, nkv, hd, splits):
             assert torch.allclose(got, want, **tol(torch.bfloat16)), (window, again)
 
 
+@pytest.mark.parametrize("nq,nkv,hd", [(8, 4, 256), (6, 1, 48), (3, 3, 80), (16, 1, 32), (4, 2, 128), (5, 5, 240)])
+@pytest.mark.parametrize("window", [None, 100, 1024])
+def test_paged_attention_mfma_merged_inside_the_block(nq, nkv, hd, window):
+    """A tile's key splits as the eight waves of one block, merged through
+    LDS: decoded tokens and portions of two and three at contexts from one
+    key (seven waves without any) to over a thousand, with and without a
+    window; the same as with the splits merged by the second kernel."""
+    portions = [(0, 1), (5, 1), (31, 2), (32, 1), (700, 1), (1210, 3), (255, 1), (1100, 1), (64, 2)]
+    if 8 * 3 * (nq // nkv) * (hd + 2) * 4 > 64 * 1024:
+        portions = [(s, 1) for s, _ in portions]  # as many columns of a tile as fit the block's LDS
+    case = Case(portions, nq, nkv, hd, 16, torch.bfloat16, 19, window)
+    want = case.reference(hd ** -0.5).float()
+    got = case.run("mfma", hd ** -0.5, prefill_kernel=False, in_block=True).float()
+    assert torch.allclose(got, want, **tol(torch.bfloat16))
+    apart = case.run("mfma", hd ** -0.5, prefill_kernel=False, in_block=False).float()
+    assert torch.allclose(got, apart, **tol(torch.bfloat16))
+
+
+def test_paged_attention_mfma_merges_inside_the_block_when_the_tiles_fill_the_machine():
+    """Seventy decoded tokens over four key/value heads are 280 tiles: the plan, left to itself, takes the kernel
+    that merges in its block; with eight requests it splits the keys over more waves."""
+    portions = [(40 + 13 * i, 1) for i in range(70)]
+    case = Case(portions, 8, 4, 128, 16, torch.bfloat16, 22, None)
+    assert ops.plan_attention_in_block(1, case.step.max_context, 2, None, 128, num_tiles=280) is not None
+    assert ops.plan_attention_in_block(1, case.step.max_context, 2, None, 128, num_tiles=32) is None
+    want = case.reference(128 ** -0.5).float()
+    assert torch.allclose(case.run("mfma", 128 ** -0.5).float(), want, **tol(torch.bfloat16))
+
+
+def test_paged_attention_mfma_merges_inside_the_block_only_what_fits():
+    case = Case([(1700, 1)], 8, 4, 256, 16, torch.bfloat16, 20)  # 54 blocks of 32 keys: seven a wave
+    with pytest.raises(ops.KernelError, match="too many to merge inside a block"):
+        case.run("mfma", 1.0 / 16, prefill_kernel=False, in_block=True)
+    case = Case([(100, 5)], 8, 4, 256, 16, torch.bfloat16, 20)  # ten columns of 256 dimensions from eight waves
+    with pytest.raises(ops.KernelError, match="too many to merge inside a block"):
+        case.run("mfma", 1.0 / 16, prefill_kernel=False, in_block=True)
+    assert ops.plan_attention_in_block(1, 8192, 2, 1024, 256) == (160, 2)  # a decoded token under the 4B model's window
+    assert ops.plan_attention_in_block(1, 8192, 2, None, 256) is None
+
+
 def test_paged_attention_mfma_long_decode_batch():
     """Decode shapes: many requests with one token each at long, different contexts."""
     portions = [(4000 + 37 * i, 1) for i in range(9)]
