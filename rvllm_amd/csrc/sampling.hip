@@ -111,7 +111,13 @@ extern "C" int rv_argmax(hipStream_t stream, const float* logits, int rows, int 
 }
 
 // ---------------------------------------------------------------------------
-// top-K select, one block per row.
+// top-K select.  A row of 262 208 logits is cut into parts, one block each: a
+// block selects the K largest of its part (radix select over the keys
+// (value, id), most significant byte first; its part stays in the caches over
+// the passes), and one more block per row selects the K largest of the parts'
+// candidates.  The reference selects with a single block per row
+// (v3/kernels/sample_topk_f32.cu:68-117); here the first pass over a row is
+// spread over many CUs, and a step's rows over the whole machine.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ unsigned long long topk_key(float v, int i) {
   unsigned int b = __float_as_uint(v);
@@ -119,15 +125,28 @@ __device__ __forceinline__ unsigned long long topk_key(float v, int i) {
   return ((unsigned long long)b << 32) | (unsigned long long)(0xFFFFFFFFu - (unsigned int)i);
 }
 
+#define TOPK_PART 8192   // elements of a part, about
+#define TOPK_MAX_PARTS 64
+#define TOPK_MAX_K 1024
+
+// grid (parts, rows).  Block (part, row) takes the elements [part * chunk, ..) of the row's `total`; element i has
+// value vals[i] and id ids[i], or i itself where ids is null.  It writes its K largest (unordered; values times
+// 1/T where inv_temp is given) at slot (row * parts + part) * k.  The host sees to it that every part has at
+// least k elements.
 __global__ void __launch_bounds__(1024)
-topk_select_kernel(const float* __restrict__ logits, int vocab, long long row_stride, int k,
-                   const float* __restrict__ inv_temp, float* __restrict__ out_val, int* __restrict__ out_idx) {
+topk_select_kernel(const float* __restrict__ vals, const int* __restrict__ ids, long long row_stride, int total,
+                   int chunk, int k, const float* __restrict__ inv_temp, float* __restrict__ out_val,
+                   int* __restrict__ out_idx) {
   __shared__ unsigned int hist[256];
   __shared__ unsigned long long prefix_s;
   __shared__ int remaining_s;
   __shared__ int out_count;
-  const int row = blockIdx.x;
-  const float* x = logits + (size_t)row * row_stride;
+  const int row = blockIdx.y;
+  const int begin = blockIdx.x * chunk;
+  const int count = total - begin < chunk ? total - begin : chunk;
+  const float* x = vals + (size_t)row * row_stride + begin;
+  const int* id_of = ids ? ids + (size_t)row * row_stride + begin : nullptr;
+  auto key_of = [&](int i) { return topk_key(x[i], id_of ? id_of[i] : begin + i); };
 
   if (threadIdx.x == 0) {
     prefix_s = 0ull;
@@ -143,45 +162,86 @@ topk_select_kernel(const float* __restrict__ logits, int vocab, long long row_st
     const unsigned long long prefix = prefix_s;
     const int shift = byte * 8;
     const unsigned long long high_mask = byte == 7 ? 0ull : (~0ull << (shift + 8));
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-      const unsigned long long key = topk_key(x[i], i);
+    for (int i = threadIdx.x; i < count; i += blockDim.x) {
+      const unsigned long long key = key_of(i);
       if ((key & high_mask) == prefix) atomicAdd(&hist[(unsigned int)(key >> shift) & 0xFFu], 1u);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      int remaining = remaining_s;
-      int bin = 255;
-      for (; bin > 0; --bin) {
-        const int c = (int)hist[bin];
-        if (c >= remaining) break;
-        remaining -= c;
+    // The bin in which the count from the top reaches `remaining`: the first wave looks, four bins a lane.
+    if (threadIdx.x < RV_WAVE) {
+      const int lane = threadIdx.x;
+      const int remaining = remaining_s;
+      int c[4], mine = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        c[j] = (int)hist[lane * 4 + j];
+        mine += c[j];
       }
-      prefix_s = prefix | ((unsigned long long)bin << shift);
-      remaining_s = remaining;
+      int from_here_up = mine;  // keys in this lane's bins and all higher ones
+#pragma unroll
+      for (int off = 1; off < RV_WAVE; off <<= 1) {
+        const int t = __shfl_down(from_here_up, off, RV_WAVE);
+        if (lane + off < RV_WAVE) from_here_up += t;
+      }
+      const int above = from_here_up - mine;
+      if (above < remaining && remaining <= from_here_up) {  // one lane: the keys that match number at least `remaining`
+        int left = remaining - above, bin = lane * 4 + 3;
+        for (int j = 3; j > 0; --j) {
+          if (c[j] >= left) break;
+          left -= c[j];
+          --bin;
+        }
+        prefix_s = prefix | ((unsigned long long)bin << shift);
+        remaining_s = left;
+      }
     }
     __syncthreads();
   }
   const unsigned long long threshold = prefix_s;  // the K-th largest key; keys are distinct
-  const float scale = inv_temp[row];
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float v = x[i];
-    if (topk_key(v, i) >= threshold) {
+  const float scale = inv_temp ? inv_temp[row] : 1.0f;
+  const size_t out0 = ((size_t)row * gridDim.x + blockIdx.x) * k;
+  for (int i = threadIdx.x; i < count; i += blockDim.x) {
+    if (key_of(i) >= threshold) {
       const int slot = atomicAdd(&out_count, 1);
       if (slot < k) {
-        out_val[(size_t)row * k + slot] = v * scale;
-        out_idx[(size_t)row * k + slot] = i;
+        out_val[out0 + slot] = x[i] * scale;
+        out_idx[out0 + slot] = id_of ? id_of[i] : begin + i;
       }
     }
   }
 }
 
+// Parts a row is cut into; with more than one, rv_topk_select wants room for rows * parts * k candidates
+// (values and ids).
+extern "C" int rv_topk_parts(int vocab) {
+  const int parts = vocab / TOPK_PART;
+  return parts < 1 ? 1 : (parts > TOPK_MAX_PARTS ? TOPK_MAX_PARTS : parts);
+}
+
 extern "C" int rv_topk_select(hipStream_t stream, const float* logits, int rows, int vocab, long long row_stride,
-                              int k, const float* inv_temp, float* out_val, int* out_idx) {
+                              int k, const float* inv_temp, float* out_val, int* out_idx, float* cand_val,
+                              int* cand_idx) {
   RV_CHECK(rows >= 0 && vocab > 0 && row_stride >= vocab, "topk_select: bad sizes rows=%d vocab=%d", rows, vocab);
-  RV_CHECK(k >= 1 && k <= 1024 && k <= vocab, "topk_select: k=%d must be in 1..min(1024, vocab=%d)", k, vocab);
+  RV_CHECK(k >= 1 && k <= TOPK_MAX_K && k <= vocab, "topk_select: k=%d must be in 1..min(%d, vocab=%d)", k, TOPK_MAX_K,
+           vocab);
   RV_CHECK(inv_temp && out_val && out_idx, "topk_select: null argument");
   if (rows == 0) return 0;
-  topk_select_kernel<<<dim3(rows), dim3(1024), 0, stream>>>(logits, vocab, row_stride, k, inv_temp, out_val, out_idx);
-  RV_LAUNCH_CHECK("topk_select");
+  RV_CHECK(rows < 65536, "topk_select: too many rows %d", rows);
+  const int parts = rv_topk_parts(vocab);
+  if (parts == 1) {
+    topk_select_kernel<<<dim3(1, rows), dim3(1024), 0, stream>>>(logits, nullptr, row_stride, vocab, vocab, k, inv_temp,
+                                                               out_val, out_idx);
+    RV_LAUNCH_CHECK("topk_select");
+    return 0;
+  }
+  RV_CHECK(cand_val && cand_idx, "topk_select: a row in %d parts needs room for the parts' candidates", parts);
+  // parts of at least TOPK_PART - TOPK_MAX_PARTS elements each: more than k
+  const int chunk = rv_div_up(vocab, parts);
+  topk_select_kernel<<<dim3(parts, rows), dim3(1024), 0, stream>>>(logits, nullptr, row_stride, vocab, chunk, k, nullptr,
+                                                                 cand_val, cand_idx);
+  RV_LAUNCH_CHECK("topk_select (parts)");
+  topk_select_kernel<<<dim3(1, rows), dim3(1024), 0, stream>>>(cand_val, cand_idx, (long long)parts * k, parts * k,
+                                                             parts * k, k, inv_temp, out_val, out_idx);
+  RV_LAUNCH_CHECK("topk_select (candidates)");
   return 0;
 }

@@ -573,8 +573,13 @@ def topk_select(logits: torch.Tensor, k: int, inv_temp: torch.Tensor) -> tuple[t
     _need(inv_temp.dtype == torch.float32 and inv_temp.numel() == rows, "topk_select: one 1/T per row expected")
     vals = torch.empty((rows, k), dtype=torch.float32, device=logits.device)
     idx = torch.empty((rows, k), dtype=torch.int32, device=logits.device)
+    parts = library().rv_topk_parts(_c_int(vocab))
+    cand_val = cand_idx = None
+    if parts > 1:  # the parts' candidates, from which the row's are selected
+        cand_val = torch.empty((rows, parts * k), dtype=torch.float32, device=logits.device)
+        cand_idx = torch.empty((rows, parts * k), dtype=torch.int32, device=logits.device)
     _check(library().rv_topk_select(_stream(), _ptr(logits), _c_int(rows), _c_int(vocab), _c_ll(vocab), _c_int(k),
-                                    _ptr(inv_temp), _ptr(vals), _ptr(idx)))
+                                    _ptr(inv_temp), _ptr(vals), _ptr(idx), _ptr(cand_val), _ptr(cand_idx)))
     return vals, idx
 
 

@@ -15,6 +15,7 @@ from __future__ import annotations
 import math
 from typing import Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..kernels import ops
@@ -79,6 +80,52 @@ def sample_from_candidates(cands: Sequence[tuple[float, int]], top_k: int, top_p
     return pool[cut - 1][1]
 
 
+def sample_rows(vals: np.ndarray, ids: np.ndarray, top_k: Sequence[int], top_p: Sequence[float],
+                rngs: Sequence[SplitMix64], vocab: Optional[int] = None) -> list[int]:
+    """``sample_from_candidates`` for many rows at once: row r has the candidates
+    (vals[r, j], ids[r, j]) and its own ``top_k``, ``top_p`` and stream.  The
+    same arithmetic in the same order, so the same tokens bit for bit, with the
+    sorting, the running sums and the walk along the weights done for all rows
+    together (a row at a time in Python costs more than the device's selection)."""
+    vals = np.asarray(vals, dtype=np.float64)
+    ids = np.asarray(ids, dtype=np.int64)
+    rows, k = vals.shape
+    if rows == 0:
+        return []
+    if k == 0:
+        raise SamplingError("candidates: must be non-empty")
+    if not np.isfinite(vals).all():
+        raise SamplingError("candidates: logits must be finite")
+    if any(not math.isfinite(p) or not 0.0 <= p <= 1.0 for p in top_p):
+        raise SamplingError("top_p: must be finite and in 0..=1")
+    if any(t > k for t in top_k):
+        raise SamplingError("top_k: must not exceed candidate count")
+    if vocab is not None and ((ids < 0) | (ids >= vocab)).any():
+        raise SamplingError("candidates: token ID must be below vocab")
+    order = np.lexsort((ids, -vals), axis=1)  # value descending, then id ascending
+    v = np.take_along_axis(vals, order, axis=1)
+    pool = np.take_along_axis(ids, order, axis=1)
+    n = np.array([min(k, t) if t > 0 else k for t in top_k], dtype=np.int64)
+    cols = np.arange(k)
+    inside = cols[None, :] < n[:, None]
+    # exp of the C library, as math.exp, not numpy's own (which differs in the last bit now and then)
+    diff = (v - v[:, :1])[inside]
+    w = np.zeros((rows, k), dtype=np.float64)
+    w[inside] = np.fromiter(map(math.exp, diff.tolist()), dtype=np.float64, count=diff.size)
+    cum = np.cumsum(w, axis=1)  # left to right, as the reference sums
+    total = cum[np.arange(rows), n - 1]
+    p = np.asarray(top_p, dtype=np.float64)
+    reached = (cum >= (np.maximum(p, 0.0) * total)[:, None]) & inside
+    cut = np.where(p < 1.0, reached.argmax(axis=1) + 1, n)
+    z = cum[np.arange(rows), cut - 1]
+    u = np.array([rng.next_f64() for rng in rngs], dtype=np.float64) * z
+    # u - w0 - w1 - ..., one subtraction after the other, as the reference walks
+    left = np.subtract.accumulate(np.concatenate([u[:, None], w], axis=1), axis=1)[:, 1:]
+    stops = (left <= 0.0) & (cols[None, :] < cut[:, None])
+    chosen = np.where(stops.any(axis=1), stops.argmax(axis=1), cut - 1)
+    return pool[np.arange(rows), chosen].tolist()
+
+
 class Sampler:
     """Next tokens for the rows of a step's logits."""
 
@@ -110,10 +157,10 @@ class Sampler:
                 inv_t = torch.tensor([1.0 / params[r].temperature for r in group], dtype=torch.float32,
                                      device=logits.device)
                 vals, ids = ops.topk_select(sub.contiguous(), k, inv_t)
-                vals, ids = vals.cpu().tolist(), ids.cpu().tolist()
-                for j, r in enumerate(group):
-                    out[r] = sample_from_candidates(list(zip(vals[j], ids[j])), params[r].top_k, params[r].top_p,
-                                                    rngs[r], self.vocab_size)
+                tokens = sample_rows(vals.cpu().numpy(), ids.cpu().numpy(), [params[r].top_k for r in group],
+                                     [params[r].top_p for r in group], [rngs[r] for r in group], self.vocab_size)
+                for r, token in zip(group, tokens):
+                    out[r] = token
         if greedy:
             host = greedy_ids.cpu().tolist()
             for r in greedy:

@@ -651,7 +651,8 @@ def test_argmax_golden_rows_of_the_reference():
     assert ops.argmax(dev(torch.tensor([[0.1, 0.2, 9.9, 0.3], [7.0, 0.0, 1.0, 2.0]]))).cpu().tolist() == [2, 0]
 
 
-@pytest.mark.parametrize("vocab,k", [(509, 509), (300, 1), (4097, 50), (262208, 1024)])
+@pytest.mark.parametrize("vocab,k", [(509, 509), (300, 1), (4097, 50), (262208, 1024), (262208, 50), (16385, 1024),
+                                     (70001, 64)])  # the row in one part, in 32, in two of which the last is the shorter
 def test_topk_select(vocab, k):
     g = torch.Generator().manual_seed(13)
     x = torch.randn(2, vocab, generator=g)

@@ -100,3 +100,50 @@ def test_params():
     assert SamplingParams(0.8, 50).kernel_k(262208) == 50
     with pytest.raises(SamplingError):
         SamplingParams(0.8, 300).kernel_k(256)
+
+
+def test_rows_drawn_together_give_what_each_gives_alone():
+    """The draw for many rows at once against the draw for one: the same tokens, and each stream advanced by one
+    number, for candidates with equal values, every cut of top_k and top_p, and one to a thousand candidates."""
+    import numpy as np
+
+    from rvllm_amd.sampling.sampler import sample_rows
+
+    gen = np.random.default_rng(3)
+    for k in (1, 2, 7, 50, 1024):
+        rows = 40
+        vals = (gen.standard_normal((rows, k)) * 3).astype(np.float32)
+        vals[::3] = np.round(vals[::3])  # many equal values: the lower id goes first
+        ids = np.stack([gen.permutation(5000)[:k] for _ in range(rows)]).astype(np.int32)
+        top_k = [int(gen.integers(0, k + 1)) for _ in range(rows)]
+        top_p = [float(x) for x in gen.choice([0.0, 0.1, 0.5, 0.9, 0.999, 1.0], size=rows)]
+        for seed in range(3):
+            together = sample_rows(vals, ids, top_k, top_p, [SplitMix64(seed * 100 + r) for r in range(rows)], 5000)
+            streams = [SplitMix64(seed * 100 + r) for r in range(rows)]
+            alone = [sample_from_candidates(list(zip(vals[r].tolist(), ids[r].tolist())), top_k[r], top_p[r], streams[r],
+                                            5000) for r in range(rows)]
+            assert together == alone, (k, seed)
+    # each stream moves by exactly one number
+    a, b = SplitMix64(9), SplitMix64(9)
+    sample_rows(np.array([[0.5, 1.5]], dtype=np.float32), np.array([[3, 4]], dtype=np.int32), [0], [1.0], [a])
+    b.next_f64()
+    assert a.next_u64() == b.next_u64()
+
+
+def test_rows_drawn_together_refuse_what_one_row_refuses():
+    import numpy as np
+
+    from rvllm_amd.sampling.sampler import sample_rows
+
+    one = lambda v, i, tk=0, tp=1.0, vocab=None: sample_rows(np.array([v], dtype=np.float32), np.array([i], dtype=np.int32),
+                                                           [tk], [tp], [SplitMix64(1)], vocab)
+    for v in ([1.0, math.nan], [math.inf, 0.0]):
+        with pytest.raises(SamplingError, match="finite"):
+            one(v, [1, 2])
+    with pytest.raises(SamplingError, match="top_k"):
+        one([1.0], [1], tk=2)
+    with pytest.raises(SamplingError, match="top_p"):
+        one([1.0], [1], tp=math.nan)
+    with pytest.raises(SamplingError, match="below vocab"):
+        one([1.0], [8], vocab=8)
+    assert one([1.0], [7], vocab=8) == [7]
