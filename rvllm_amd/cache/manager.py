@@ -60,6 +60,32 @@ class PageGroup:
         return max(0, need - len(table))
 
 
+class Reservation:
+    """The pages that the portions planned for a step will take, summed as
+    they are planned, so that asking whether one more fits costs that one's
+    own count and not everyone's again.  ``fits`` and then ``add`` say what
+    ``CacheManager.can_extend`` says for the whole list so far: the pools are
+    read as they are when asked, so pages that a set-back request gave back in
+    between count as free.  A request that is not live needs a free slot;
+    once planned it is expected to be made live at once (its slot then leaves
+    the free ones), so only the one asked about can be new."""
+
+    def __init__(self, cache: "CacheManager"):
+        self.cache = cache
+        self.pages = {name: 0 for name in cache.groups}
+
+    def fits(self, request: Hashable, new_length: int) -> bool:
+        cache = self.cache
+        if request not in cache.requests and cache.slots.free_count < 1:
+            return False
+        need = cache.pages_needed(request, new_length)
+        return all(self.pages[name] + n <= cache.groups[name].pool.free_count for name, n in need.items())
+
+    def add(self, request: Hashable, new_length: int) -> None:
+        for name, n in self.cache.pages_needed(request, new_length).items():
+            self.pages[name] += n
+
+
 class CacheManager:
     def __init__(self, needs: Sequence, page_size: int, num_pages, max_requests: int):
         """``needs[i]`` is layer i's need (KVNeed, StateNeed or None).
@@ -133,6 +159,10 @@ class CacheManager:
         except OutOfPages:
             return False
         return True
+
+    def reservation(self) -> "Reservation":
+        """An empty tally of what a step's planned portions will take."""
+        return Reservation(self)
 
     def extend(self, request: Hashable, new_length: int) -> None:
         """Give the request pages for the positions up to ``new_length``

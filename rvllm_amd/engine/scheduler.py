@@ -131,17 +131,17 @@ class Scheduler:
     def schedule(self) -> StepPlan:
         budget = self.max_num_batched_tokens
         portions: list[PlannedPortion] = []
-        planned: list[tuple[Hashable, int]] = []  # (request id, length after this step)
+        reserved = self.cache.reservation()  # the pages that the portions planned so far will take
         set_back: list[Request] = []
         ended: list[Request] = []
 
         def fits(req: Request, new_len: int) -> bool:
-            return self.cache.can_extend(planned + [(req.id, new_len)])
+            return reserved.fits(req.id, new_len)
 
         def take(req: Request, count: int) -> None:
             nonlocal budget
             portions.append(PlannedPortion(req, req.computed, count, req.computed + count == req.total))
-            planned.append((req.id, req.computed + count))
+            reserved.add(req.id, req.computed + count)
             budget -= count
 
         # Requests that are decoding come first, then prompts under way; both
@@ -153,13 +153,15 @@ class Scheduler:
                 continue  # set back while an earlier request was planned, or no budget left
             left = req.total - req.computed
             count = min(left, self.max_prefill_chunk if left > 1 else 1, budget)
-            while not fits(req, req.computed + count):
+            room = fits(req, req.computed + count)
+            while not room:
                 victim = self._latest_running(exclude_planned={p.request.id for p in portions})
                 if victim is None or victim is req:
                     break
                 self._set_back(victim)
                 set_back.append(victim)
-            if fits(req, req.computed + count):
+                room = fits(req, req.computed + count)
+            if room:
                 take(req, count)
             elif self._runs_alone(req, portions):
                 # nothing else holds pages and it still does not fit

@@ -88,6 +88,48 @@ def test_out_of_pages_takes_nothing():
     m.check()
 
 
+def test_a_reservation_says_what_the_whole_list_says():
+    """The tally a scheduler keeps while it plans a step: asked one request at a time, it answers as
+    ``can_extend`` does for everything planned so far and the one more, for live requests and new ones, with pools
+    that run out of pages and of slots, and after a request that was not planned gave its pages back in between."""
+    rng = random.Random(5)
+    refused = accepted = 0
+    for trial in range(80):
+        m = make(num_pages=rng.choice([6, 10, 24]), page_size=4, max_requests=rng.choice([3, 6]))
+        live = []
+        for i in range(rng.randrange(0, 4)):
+            length = rng.randrange(1, 14)
+            if m.can_extend([(f"old{i}", length)]):
+                m.add_request(f"old{i}")
+                m.extend(f"old{i}", length)
+                m.commit(f"old{i}", length)
+                live.append(f"old{i}")
+        tally, planned = m.reservation(), []
+        candidates = [(rid, m.length(rid) + rng.randrange(1, 30)) for rid in live] + \
+                     [(f"new{j}", rng.randrange(1, 30)) for j in range(5)]
+        rng.shuffle(candidates)
+        gone = set()
+        for rid, new_len in candidates:
+            if rid in gone:
+                continue
+            want = m.can_extend(planned + [(rid, new_len)])
+            assert tally.fits(rid, new_len) == want, (trial, rid, new_len)
+            if want:
+                accepted += 1
+                if not m.has_request(rid):
+                    m.add_request(rid)  # as a scheduler admits what it has planned
+                tally.add(rid, new_len)
+                planned.append((rid, new_len))
+            else:
+                refused += 1
+                unplanned = [r for r in live if r not in gone and all(r != p for p, _ in planned)]
+                if unplanned and rng.random() < 0.5:
+                    m.release(unplanned[-1])  # set back: its pages count as free from now on
+                    gone.add(unplanned[-1])
+        m.check()
+    assert refused > 20 and accepted > 20
+
+
 def test_commit_without_pages_is_caught():
     m = make()
     m.add_request("a")
