@@ -178,6 +178,27 @@ class CacheManager:
             if n:
                 rc.tables[name].extend(self.groups[name].pool.take(request, n))
 
+    def extend_all(self, wanted: Sequence[tuple[Hashable, int]]) -> None:
+        """``extend`` for every (live request, new length) of a step: all of
+        them get their pages or, with OutOfPages, none does."""
+        needs = []
+        total = {name: 0 for name in self.groups}
+        for request, new_length in wanted:
+            rc = self.requests[request]
+            if new_length < rc.length:
+                raise ValueError(f"request {request!r} holds {rc.length} tokens, cannot extend to {new_length}")
+            need = self.pages_needed(request, new_length)
+            needs.append((rc, need))
+            for name, n in need.items():
+                total[name] += n
+        for name, g in self.groups.items():
+            if total[name] > g.pool.free_count:
+                raise OutOfPages(name, total[name], g.pool.free_count)
+        for rc, need in needs:
+            for name, n in need.items():
+                if n:
+                    rc.tables[name].extend(self.groups[name].pool.take(rc.request, n))
+
     def adopt_length(self, request: Hashable, length: int) -> None:
         """Make a fresh request hold ``length`` tokens without running them:
         it gets exactly the pages a request of that length holds (none behind

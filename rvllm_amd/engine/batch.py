@@ -134,38 +134,47 @@ class BatchBuilder:
             raise ValueError(f"step has {T} tokens, the engine was built for {lay.max_tokens}")
         tok, pos, req, rows = (self._host(n) for n in ("token_ids", "positions", "token_req", "logit_rows"))
         qs, cs, cl, ss = (self._host(n) for n in ("q_start", "chunk_start", "context_len", "state_slot"))
-        t = 0
-        r = 0
-        max_portion = 1
-        max_context = 1
+        # Whole arrays at a time, not a portion at a time: with 64 decoded tokens a step, a handful of small
+        # assignments per portion cost the host more than the step costs the GPU.
+        lens = np.fromiter((len(p.tokens) for p in portions), dtype=np.int64, count=B)
+        if B and lens.min() < 1:
+            raise ValueError("a portion must hold at least one token")
+        starts = np.fromiter((p.start for p in portions), dtype=np.int64, count=B)
+        first = np.zeros(B + 1, dtype=np.int64)  # first token of each portion
+        np.cumsum(lens, out=first[1:])
+        tok[:T] = np.concatenate([np.asarray(p.tokens, dtype=np.int32) for p in portions]) if T else 0
+        req[:T] = np.repeat(np.arange(B, dtype=np.int32), lens)
+        pos[:T] = np.arange(T, dtype=np.int64) + np.repeat(starts - first[:B], lens)
+        qs[: B + 1] = first
+        cs[:B] = starts
+        cl[:B] = starts + lens
+        ss[:B] = np.fromiter(state_slots, dtype=np.int64, count=B)
+        wanted = []
         for b, p in enumerate(portions):
-            n = len(p.tokens)
-            if n < 1:
-                raise ValueError("a portion must hold at least one token")
-            tok[t : t + n] = np.asarray(p.tokens, dtype=np.int32)
-            pos[t : t + n] = np.arange(p.start, p.start + n, dtype=np.int32)
-            req[t : t + n] = b
+            n, t = int(lens[b]), int(first[b])
             for wplace in p.want:
                 if not 0 <= wplace < n:
                     raise ValueError(f"wanted place {wplace} outside a portion of {n} tokens")
-                rows[r] = t + wplace
-                r += 1
-            qs[b] = t
-            cs[b] = p.start
-            cl[b] = p.start + n
-            ss[b] = state_slots[b]
-            max_portion = max(max_portion, n)
-            max_context = max(max_context, p.start + n)
-            t += n
-        qs[B] = T
+                wanted.append(t + wplace)
+        r = len(wanted)
+        rows[:r] = wanted
+        max_portion = max(1, int(lens.max())) if B else 1
+        max_context = max(1, int((starts + lens).max())) if B else 1
         for name, width in lay.table_widths.items():
             off, _ = lay.offsets["bt:" + name]
-            dst = self.host_np[off : off + B * width].reshape(B, width)
+            dst = self.host_np[off : off + B * width]
             dst.fill(-1)
-            for b, row in enumerate(tables[name]):
-                if len(row) > width:
-                    raise ValueError(f"block table of group {name} has {len(row)} entries, width is {width}")
-                dst[b, : len(row)] = row
+            held = [np.asarray(row, dtype=np.int32) for row in tables[name]]
+            counts = np.fromiter((len(row) for row in held), dtype=np.int64, count=B)
+            if B and counts.max() > width:
+                raise ValueError(f"block table of group {name} has {int(counts.max())} entries, width is {width}")
+            total = int(counts.sum())
+            if total:
+                # entry j of row b goes to b * width + j
+                row_first = np.zeros(B, dtype=np.int64)
+                np.cumsum(counts[:-1], out=row_first[1:])
+                where = np.arange(total, dtype=np.int64) + np.repeat(np.arange(B, dtype=np.int64) * width - row_first, counts)
+                dst[where] = np.concatenate(held)
         self.dev.copy_(self.host, non_blocking=True)
         if event is not None:
             event.record()

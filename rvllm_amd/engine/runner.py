@@ -207,12 +207,11 @@ class ModelRunner:
             ids = np.asarray(tokens, dtype=np.int64)
             if ids.ndim != 1 or ids.size == 0:
                 raise ValueError(f"request {request!r}: a portion must hold at least one token")
-            if ids.min() < 0 or ids.max() >= vocab:
+            low, high = (int(ids[0]),) * 2 if ids.size == 1 else (int(ids.min()), int(ids.max()))
+            if low < 0 or high >= vocab:
                 raise ValueError(f"request {request!r}: token id outside the vocabulary of {vocab}")
             portions.append(Portion(request, ids, start, want))
-        self.cache.require([(p.request, p.start + len(p.tokens)) for p in portions])
-        for p in portions:
-            self.cache.extend(p.request, p.start + len(p.tokens))
+        self.cache.extend_all([(p.request, p.start + len(p.tokens)) for p in portions])
         tables = {name: [self.cache.table(p.request, name) for p in portions] for name in self.cache.groups}
         batch = self.builder.build(portions, tables, [self.cache.slot(p.request) for p in portions])
         logits = self._forward(batch)

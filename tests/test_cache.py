@@ -88,6 +88,26 @@ def test_out_of_pages_takes_nothing():
     m.check()
 
 
+def test_a_step_gets_all_its_pages_or_none():
+    m = make(num_pages=6, page_size=4)
+    for rid in "abc":
+        m.add_request(rid)
+    m.extend_all([("a", 8), ("b", 5), ("c", 1)])  # 2 + 2 + 1 pages of 6
+    assert [len(m.table(r, "full")) for r in "abc"] == [2, 2, 1]
+    for rid, n in (("a", 8), ("b", 5), ("c", 1)):
+        m.commit(rid, n)
+    with pytest.raises(OutOfPages):
+        m.extend_all([("a", 9), ("b", 9)])  # one page each, one is left
+    assert [len(m.table(r, "full")) for r in "abc"] == [2, 2, 1] and m.free_pages()["full"] == 1
+    with pytest.raises(ValueError, match="cannot extend"):
+        m.extend_all([("a", 7)])
+    with pytest.raises(KeyError):
+        m.extend_all([("nobody", 1)])
+    m.extend_all([("c", 4), ("a", 9)])  # c needs none
+    assert m.free_pages()["full"] == 0
+    m.check()
+
+
 def test_a_reservation_says_what_the_whole_list_says():
     """The tally a scheduler keeps while it plans a step: asked one request at a time, it answers as
     ``can_extend`` does for everything planned so far and the one more, for live requests and new ones, with pools
