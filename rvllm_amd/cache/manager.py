@@ -73,17 +73,24 @@ class Reservation:
     def __init__(self, cache: "CacheManager"):
         self.cache = cache
         self.pages = {name: 0 for name in cache.groups}
+        self._asked = None  # (request, new length, its pages): `add` usually follows `fits` for the same
+
+    def _need(self, request: Hashable, new_length: int) -> dict[str, int]:
+        if self._asked is None or self._asked[0] != request or self._asked[1] != new_length:
+            self._asked = (request, new_length, self.cache.pages_needed(request, new_length))
+        return self._asked[2]
 
     def fits(self, request: Hashable, new_length: int) -> bool:
         cache = self.cache
         if request not in cache.requests and cache.slots.free_count < 1:
             return False
-        need = cache.pages_needed(request, new_length)
+        need = self._need(request, new_length)
         return all(self.pages[name] + n <= cache.groups[name].pool.free_count for name, n in need.items())
 
     def add(self, request: Hashable, new_length: int) -> None:
-        for name, n in self.cache.pages_needed(request, new_length).items():
+        for name, n in self._need(request, new_length).items():
             self.pages[name] += n
+        self._asked = None
 
 
 class CacheManager:
