@@ -1,5 +1,5 @@
 """The engine at the layer sizes of the 4B model (two layers, a small
-vocabulary) against the plain implementation: sequences that cross the edge of
+vocabulary), and with the heads of the 27B model, against the plain implementation: sequences that cross the edge of
 the window of 1024, whole, with the last tokens decoded one by one, in large
 and small portions, and two requests mixed.  What the tiny configurations
 cannot show lies here: portions of more than a thousand tokens (the library's
@@ -20,9 +20,10 @@ pytestmark = pytest.mark.gpu
 LENGTHS = [1300, 700]
 
 
-@pytest.fixture(scope="module")
-def model(tmp_path_factory):
-    folder = tiny_models.write_model(tmp_path_factory.mktemp("larger") / "D", "D")
+@pytest.fixture(scope="module", params=["D", "E"])
+def model(request, tmp_path_factory):
+    """D: two layers of the 4B model's sizes.  E: three narrow layers with the 27B model's heads."""
+    folder = tiny_models.write_model(tmp_path_factory.mktemp("larger") / request.param, request.param)
     weights, cfg = plain_gemma.load_weights(folder), plain_gemma.read_config(folder)
     seqs = tt.make_sequences(cfg["vocab"], LENGTHS, seed=4)
     refs = {rid: plain_gemma.forward(weights, cfg, ids, torch.float64) for rid, ids in seqs.items()}

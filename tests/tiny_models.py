@@ -108,8 +108,32 @@ CONFIG_D = {
     "final_logit_softcapping": None,
 }
 
+# The head geometry of the 27B model (32 query heads on 16 key/value heads of 128 dimensions, scores scaled by
+# 168^-1/2, not by the head size) on a narrow layer: three layers, the global one in the middle.
+CONFIG_E = {
+    "architectures": ["Gemma3ForCausalLM"],
+    "num_hidden_layers": 3,
+    "layer_types": ["sliding_attention", "full_attention", "sliding_attention"],
+    "hidden_size": 672,
+    "num_attention_heads": 32,
+    "num_key_value_heads": 16,
+    "head_dim": 128,
+    "intermediate_size": 1344,
+    "vocab_size": 811,
+    "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 8192,
+    "sliding_window": 1024,
+    "rope_theta": 1000000.0,
+    "rope_local_base_freq": 10000.0,
+    "rope_scaling": {"rope_type": "linear", "factor": 8.0},
+    "query_pre_attn_scalar": 168,
+    "hidden_activation": "gelu_pytorch_tanh",
+    "tie_word_embeddings": True,
+    "final_logit_softcapping": None,
+}
+
 CONFIGS = {"A": (CONFIG_A, 0), "B": (CONFIG_B, 1), "C": (CONFIG_C, 2)}
-LARGER = {"D": (CONFIG_D, 3)}
+LARGER = {"D": (CONFIG_D, 3), "E": (CONFIG_E, 4)}
 
 
 def write_model(folder, name: str, dtype=torch.bfloat16, seed=None) -> Path:
