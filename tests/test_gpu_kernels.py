@@ -726,3 +726,35 @@ def test_sliced_product_through_the_skinny_kernel():
     want = x.double() @ w.double().T
     assert torch.allclose(got.as_tensor().cpu().double(), want, atol=3e-2, rtol=2e-2)
     assert torch.allclose(got.data.sum(0).cpu().double(), want, atol=1e-3, rtol=1e-4)
+
+
+def test_sampler_at_a_large_vocabulary_draws_what_one_row_alone_draws():
+    """Rows that are greedy, that sample with different temperatures, cuts and seeds, and rows with many equal
+    logits, over a vocabulary that the selection cuts into 32 parts: each row's token is the one that the single
+    row's draw gives from that row's exact top candidates."""
+    from rvllm_amd.sampling.params import SamplingParams
+    from rvllm_amd.sampling.sampler import Sampler, SplitMix64, sample_from_candidates
+
+    vocab = 262208
+    g = torch.Generator().manual_seed(23)
+    logits = torch.randn(7, vocab, generator=g) * 2.0
+    logits[3] = torch.round(logits[3])       # many equal values: lower ids first among them
+    logits[5, 1000:200000] = 3.5
+    params = [SamplingParams(), SamplingParams(0.8, 50, 1.0, seed=1), SamplingParams(1.3, 50, 0.9, seed=2),
+              SamplingParams(0.7, 7, 0.5, seed=3), SamplingParams(1.0, 1024, 0.95, seed=4),
+              SamplingParams(0.9, 50, 1.0, seed=5), SamplingParams(0.8, 50, 0.0, seed=6)]
+    sampler = Sampler(vocab)
+    for trial in range(3):
+        rngs = [SplitMix64(100 * trial + i) for i in range(7)]
+        got = sampler.sample(dev(logits), params, rngs)
+        for r, p in enumerate(params):
+            row = logits[r]
+            if p.is_greedy():
+                assert got[r] == int(row.argmax())
+                continue
+            k = p.kernel_k(vocab)
+            order = sorted(range(vocab), key=lambda i: (-row[i].item(), i))[:k] if r in (3, 5) else \
+                torch.topk(row, k).indices.tolist()
+            cands = [((row[i] * torch.tensor(1.0 / p.temperature)).item(), i) for i in order]
+            want = sample_from_candidates(cands, p.top_k, p.top_p, SplitMix64(100 * trial + r), vocab)
+            assert got[r] == want, (trial, r)
