@@ -9,6 +9,7 @@ trace replay all go through it.
 
 from __future__ import annotations
 
+import collections
 import dataclasses
 import os
 from typing import Hashable, Optional, Sequence
@@ -60,13 +61,14 @@ class ModelRunner:
         self.builder = BatchBuilder(self.device, cfg.max_num_batched_tokens, cfg.max_num_seqs,
                                     {name: width for name in self.cache.groups})
         # Captured decode steps, by (requests, context bucket).
-        self._graphs: dict[tuple[int, int], tuple] = {}
+        self._graphs: collections.OrderedDict[tuple[int, int], tuple] = collections.OrderedDict()
         self._graph_pool = None
         self.graph_replays = 0
 
     # ---- decode steps from captured graphs -------------------------------
     GRAPH_CONTEXT_BUCKET = 1024
     GRAPH_MAX_REQUESTS = 64  # beyond this the products go to the library, which stays out of graphs
+    GRAPH_MAX_KEPT = 128     # shapes whose graphs are kept; the one unused for longest goes first
 
     def _graph_key(self, batch: StepBatch):
         """The key of the captured graph that can run this batch, or None.
@@ -101,7 +103,10 @@ class ModelRunner:
             if self._graph_pool is None:
                 self._graph_pool = graph.pool()
             self._graphs[key] = (graph, static_logits)
+            while len(self._graphs) > self.GRAPH_MAX_KEPT:
+                self._graphs.popitem(last=False)
             return logits
+        self._graphs.move_to_end(key)
         graph, static_logits = entry
         graph.replay()
         self.graph_replays += 1

@@ -163,6 +163,33 @@ def test_decode_steps_replayed_from_a_graph_match_eager_steps(model_dirs, plain_
     assert len(graph._graphs) >= 2
 
 
+def test_a_graph_dropped_for_room_is_recorded_again(model_dirs, plain_models):
+    """Only so many shapes keep their graphs.  With room for one, a shape that comes back after another was met
+    runs eagerly once more, is recorded again and replayed, with right logits all the way."""
+    weights, cfg = plain_models["A"]
+    runner = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(
+        dtype="bfloat16", max_model_len=256, max_num_seqs=4, max_num_batched_tokens=64, max_prefill_chunk=64,
+        max_cache_tokens=1024, use_graphs=True)).runner
+    runner.GRAPH_MAX_KEPT = 1
+    seqs = tt.make_sequences(cfg["vocab"], [60, 60, 60], seed=9)
+    refs = {rid: plain_gemma.forward(weights, cfg, ids, torch.float64) for rid, ids in seqs.items()}
+    for rid, ids in seqs.items():
+        runner.add_request(rid)
+        runner.step([(rid, ids[:10], [])])
+    done = {rid: 10 for rid in seqs}
+    replays = []
+    for it in range(15):
+        live = list(seqs) if (it // 5) % 2 == 0 else list(seqs)[:2]  # three requests, two, three again
+        before = runner.graph_replays
+        got = runner.step([(rid, [seqs[rid][done[rid]]], [0]) for rid in live]).float().cpu()
+        replays.append(runner.graph_replays - before)
+        for row, rid in enumerate(live):
+            tt.compare(got[row:row + 1].numpy(), refs[rid][done[rid]:done[rid] + 1], "bfloat16", f"step {it} {rid}")
+            done[rid] += 1
+        assert len(runner._graphs) == 1
+    assert replays == [0, 1, 1, 1, 1] * 3  # the first step of each run of a shape is eager
+
+
 def test_eos_and_capacity_reasons(model_dirs):
     engine = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(dtype="float32", max_model_len=128,
                                                                     max_num_seqs=2, max_cache_tokens=32))
