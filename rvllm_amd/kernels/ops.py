@@ -94,7 +94,9 @@ def _i32(*tensors: torch.Tensor) -> None:
         _need(t.dtype == torch.int32, f"index tensors must be int32, got {t.dtype}")
 
 
-_c_int, _c_float, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_longlong
+# A Python int goes to a foreign function as a C int by itself; making a ctypes object for each of the twenty-odd
+# sizes of a launch costs more than the rest of the call.  Floats, 64-bit numbers and addresses keep their types.
+_c_int, _c_float, _c_ll = int, ctypes.c_float, ctypes.c_longlong
 
 
 def _cache_geometry(k_pages: torch.Tensor, v_pages: torch.Tensor, what: str) -> tuple[int, int, int, int]:
