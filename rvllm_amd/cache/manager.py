@@ -137,10 +137,13 @@ class CacheManager:
     def pages_needed(self, request: Hashable, new_length: int) -> dict[str, int]:
         """Pages each group must add so that the request can hold ``new_length`` tokens."""
         rc = self.requests.get(request)
+        pages = -(-new_length // self.page_size)  # every group has the manager's page size
+        if rc is None:
+            return {name: pages for name in self.groups}
         out = {}
-        for name, g in self.groups.items():
-            table = rc.tables[name] if rc is not None else ()
-            out[name] = g.pages_to_add(table, new_length)
+        for name, table in rc.tables.items():
+            more = pages - len(table)
+            out[name] = more if more > 0 else 0
         return out
 
     def require(self, wanted: Sequence[tuple[Hashable, int]]) -> None:
