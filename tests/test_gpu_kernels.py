@@ -195,6 +195,36 @@ def test_gated_act_over_rows_in_fours(dtype):
         ops.gated_act(dev(torch.zeros(2, 2 * 42, dtype=dtype)), "silu", fours=True)
 
 
+@pytest.mark.parametrize("m", [1, 8, 33, 64])
+def test_gemm_skinny_under_every_plan(m):
+    """The plan (waves a block, slices of K) is chosen by a model of the machine, one per shape; here every plan is
+    forced in turn, with slices that end inside the last piece of x and blocks that reach past the last row of W."""
+    lib = ops.library()
+    g = torch.Generator().manual_seed(24)
+    n, k = 1000, 1416  # 11.06 pieces of 128 columns; 62.5 tiles of 16 rows
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    want = x.double() @ w.double().T
+    scale = want.abs().max().item()
+    try:
+        for waves in (4, 5, 6, 7, 8):
+            for per in (1, 2, 3, 5, 12):
+                lib.rv_gemm_skinny_force_plan(waves, per)
+                out = ops.gemm_bf16(dev(x), dev(w), out_dtype=torch.float32)
+                err = (out.cpu().double() - want).abs().max().item()
+                assert err <= 2e-6 * scale * max(1.0, math.sqrt(k) / 16), (waves, per)
+                # the slices handed on unreduced add up to the same bits as the product that adds them itself
+                sums = ops.gemm_bf16(dev(x), dev(w), sliced_ok=True)
+                whole = ops.gemm_bf16(dev(x), dev(w))
+                if isinstance(sums, ops.SlicedSums):
+                    assert sums.slices == -(-12 // per) and sums.slices > 1
+                    assert torch.equal(sums.as_tensor(), whole), (waves, per)
+                else:
+                    assert per == 12 and torch.equal(sums, whole)
+    finally:
+        lib.rv_gemm_skinny_force_plan(0, 0)
+
+
 def test_gemm_skinny_reads_strided_rows_and_refuses_what_it_cannot():
     g = torch.Generator().manual_seed(21)
     big = dev(torch.randn(6, 96, generator=g).bfloat16())
