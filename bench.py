@@ -121,16 +121,24 @@ def time_decode(engine_parts, batch: int, context: int, steps: int, warmup: int)
     rngs = [SplitMix64(0) for _ in ids]
     tokens = [(17 * b + 5) % runner.model.spec.vocab_size for b in range(batch)]
 
-    def one_step(tokens):
-        logits = runner.step([(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
-        return sampler.sample(logits, params, rngs)  # greedy: arg-max on the device, ids back on the host
+    ahead = runner.config.greedy_steps_ahead
 
-    for _ in range(warmup):
-        tokens = one_step(tokens)
+    def decode(count, tokens):
+        """Exactly ``count`` decode steps, as the engine runs greedy requests: up to ``ahead`` steps follow one
+        another with the chosen tokens handed on on the device, then the ids come back to the host."""
+        while count > 0:
+            if ahead > 1:
+                rows = runner.decode_greedy(list(zip(ids, tokens)), min(ahead, count))
+                tokens, count = rows[-1], count - len(rows)
+            else:
+                logits = runner.step([(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
+                tokens, count = sampler.sample(logits, params, rngs), count - 1
+        return tokens
+
+    tokens = decode(warmup, tokens)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        tokens = one_step(tokens)
+    tokens = decode(steps, tokens)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     release_all(runner, ids)
@@ -226,6 +234,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--graphs", type=int, default=1, help="replay decode steps from captured HIP graphs (0 = off)")
+    ap.add_argument("--steps-ahead", type=int, default=None,
+                    help="greedy decode steps that follow one another without the host (1 = off; default: the engine's)")
     ap.add_argument("--workload", choices=sorted(WORKLOADS), help="instead of the default run: an engine workload of a "
                     "larger configuration (requests through the scheduler); --requests and --layers shrink it")
     ap.add_argument("--requests", type=int, default=0)
@@ -255,7 +265,8 @@ def main() -> int:
         dtype=args.dtype, page_size=16, max_model_len=args.context + steps_total,
         max_num_seqs=max_batch, max_num_batched_tokens=max(args.prefill_tokens, max_batch),
         max_prefill_chunk=max(args.prefill_tokens, 1), max_cache_tokens=max_batch * (args.context + steps_total + 16),
-        use_graphs=bool(args.graphs))
+        use_graphs=bool(args.graphs),
+        **({} if args.steps_ahead is None else {"greedy_steps_ahead": args.steps_ahead}))
     log(f"building {args.layers}-layer model with random weights ({short})")
     t0 = time.time()
     runner = ModelRunner.from_random(cfg, 0, engine_cfg)
@@ -304,7 +315,7 @@ def main() -> int:
             "sliding_to_global": "5:1",
             "rope_local_global_factor": "1e4/1e6/8",
             "page_size": engine_cfg.page_size,
-            "hip_graphs": bool(args.graphs),
+            "hip_graphs": bool(args.graphs), "greedy_steps_ahead": engine_cfg.greedy_steps_ahead,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},

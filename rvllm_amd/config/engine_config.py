@@ -38,6 +38,9 @@ class EngineConfig:
     max_cache_tokens: Optional[int] = None
     # Replay decode-only steps from captured HIP graphs (bf16 only).
     use_graphs: bool = True
+    # Greedy decode steps that may follow one another without the host in between, while nothing waits to be
+    # admitted and no request can end by its length on the way (1 = every step is planned by itself).
+    greedy_steps_ahead: int = 4
 
     @property
     def torch_dtype(self) -> torch.dtype:
@@ -59,6 +62,8 @@ class EngineConfig:
             problems.append("max_prefill_chunk must be >= 1")
         if self.max_prefill_chunk > self.max_num_batched_tokens:
             problems.append("max_prefill_chunk must not exceed max_num_batched_tokens")
+        if not 1 <= self.greedy_steps_ahead <= 64:
+            problems.append(f"greedy_steps_ahead {self.greedy_steps_ahead} must be in 1..=64")
         if self.max_cache_tokens is not None and self.max_cache_tokens < self.page_size:
             problems.append("max_cache_tokens must hold at least one page")
         if problems:

@@ -245,3 +245,30 @@ extern "C" int rv_topk_select(hipStream_t stream, const float* logits, int rows,
   RV_LAUNCH_CHECK("topk_select (candidates)");
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// From one decode step to the next without the host: every request's chosen
+// token becomes its next token, one position on.  A step of decoded tokens is
+// described by these arrays alone (token t belongs to request t), so the same
+// launches, or the same captured graph, run the next step from them.
+// ---------------------------------------------------------------------------
+__global__ void advance_decode_kernel(const int* __restrict__ chosen, int* __restrict__ token_ids,
+                                      int* __restrict__ positions, int* __restrict__ chunk_start,
+                                      int* __restrict__ context_len, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  token_ids[i] = chosen[i];
+  positions[i] += 1;
+  chunk_start[i] += 1;
+  context_len[i] += 1;
+}
+
+extern "C" int rv_advance_decode(hipStream_t stream, const int* chosen, int* token_ids, int* positions,
+                                 int* chunk_start, int* context_len, int n) {
+  RV_CHECK(n >= 0 && chosen && token_ids && positions && chunk_start && context_len, "advance_decode: bad arguments");
+  if (n == 0) return 0;
+  advance_decode_kernel<<<dim3(rv_div_up(n, 256)), dim3(256), 0, stream>>>(chosen, token_ids, positions, chunk_start,
+                                                                         context_len, n);
+  RV_LAUNCH_CHECK("advance_decode");
+  return 0;
+}

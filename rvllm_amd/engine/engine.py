@@ -25,7 +25,7 @@ from ..config.engine_config import EngineConfig
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .runner import ModelRunner
-from .scheduler import Request, RequestState, Scheduler, StepPlan
+from .scheduler import PlannedPortion, Request, RequestState, Scheduler, StepPlan
 
 
 @dataclasses.dataclass
@@ -45,6 +45,7 @@ class LLMEngine:
                                    cfg.max_model_len, on_admit=self._on_admit)
         self.sampler = Sampler(runner.model.spec.vocab_size)
         self.steps = 0
+        self.plans = 0  # plans that ran something; fewer than steps when greedy steps followed one another
         self.tokens_run = 0
 
     @classmethod
@@ -85,10 +86,14 @@ class LLMEngine:
         entries = []
         wanting = []
         for p in plan.portions:
-            tokens = p.request.tokens[p.start : p.start + p.count]
+            tokens = p.request.tokens_at(p.start, p.count)
             entries.append((p.request.id, tokens, [p.count - 1] if p.wants_token else []))
             if p.wants_token:
                 wanting.append(p.request)
+        self.plans += 1
+        ahead = self._greedy_steps_ahead(plan)
+        if ahead > 1:
+            return results + self._decode_ahead(plan, ahead)
         logits = self.runner.step(entries)
         self.steps += 1
         self.tokens_run += plan.num_tokens
@@ -96,6 +101,37 @@ class LLMEngine:
         next_tokens = {r.id: t for r, t in zip(wanting, chosen)}
         finished = self.scheduler.commit(plan, next_tokens)
         return results + [self._result(r) for r in finished]
+
+    # ---- several greedy steps from one plan ------------------------------
+    def _greedy_steps_ahead(self, plan: StepPlan) -> int:
+        """How many decode steps may follow one another from this plan: more
+        than one only if every request in it decodes greedily, none could end
+        by its length or the model's on the way, nothing was set back, and no
+        request waits (it would be admitted that much later).  A request that
+        meets an end id on the way stops there; what was run for it after
+        that is dropped, and costs the others nothing."""
+        ahead = self.runner.config.greedy_steps_ahead
+        if ahead <= 1 or self.scheduler.waiting or plan.set_back:
+            return 1
+        for p in plan.portions:
+            req = p.request
+            if p.count != 1 or not p.wants_token or not req.params.is_greedy():
+                return 1
+            ahead = min(ahead, req.max_new_tokens - len(req.output), self.scheduler.max_model_len - req.total)
+        return max(1, ahead)
+
+    def _decode_ahead(self, plan: StepPlan, ahead: int) -> list[GenerationResult]:
+        rows = self.runner.decode_greedy([(p.request.id, p.request.tokens_at(p.start, 1)[0]) for p in plan.portions], ahead)
+        finished: list[Request] = []
+        for i, row in enumerate(rows):
+            live = [(p, token) for p, token in zip(plan.portions, row) if p.request.state is RequestState.RUNNING]
+            if not live:
+                break
+            self.steps += 1
+            self.tokens_run += len(live)
+            step_plan = StepPlan([PlannedPortion(p.request, p.start + i, 1, True) for p, _ in live], [], [])
+            finished += self.scheduler.commit(step_plan, {p.request.id: token for p, token in live})
+        return [self._result(r) for r in finished]
 
     @staticmethod
     def _result(req: Request) -> GenerationResult:

@@ -79,12 +79,16 @@ class ModelRunner:
         is made for that end; splits past a request's own context are empty).
         The reference captures its decode step the same way, once per batch
         size (v3/crates/rvllm-runtime/src/gemma4_serve.rs:594-694)."""
-        if not (self.config.use_graphs and self.dtype == torch.bfloat16 and batch.decode_only):
+        if not batch.decode_only or batch.num_logit_rows != batch.num_tokens:
             return None
-        if batch.num_logit_rows != batch.num_tokens or batch.num_requests > self.GRAPH_MAX_REQUESTS:
+        return self._decode_graph_key(batch.num_requests, batch.max_context)
+
+    def _decode_graph_key(self, num_requests: int, max_context: int):
+        """The key for a step of ``num_requests`` decoded tokens, all wanted, at contexts up to ``max_context``."""
+        if not (self.config.use_graphs and self.dtype == torch.bfloat16) or num_requests > self.GRAPH_MAX_REQUESTS:
             return None
-        bucket = -(-batch.max_context // self.GRAPH_CONTEXT_BUCKET) * self.GRAPH_CONTEXT_BUCKET
-        return batch.num_requests, bucket
+        bucket = -(-max_context // self.GRAPH_CONTEXT_BUCKET) * self.GRAPH_CONTEXT_BUCKET
+        return num_requests, bucket
 
     def _forward(self, batch: StepBatch) -> torch.Tensor:
         key = self._graph_key(batch)
@@ -198,6 +202,15 @@ class ModelRunner:
         tokens."""
         if not entries:
             return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32, device=self.device)
+        portions = self._portions(entries)
+        self.cache.extend_all([(p.request, p.start + len(p.tokens)) for p in portions])
+        logits = self._forward(self._batch(portions))
+        for p in portions:
+            self.cache.commit(p.request, p.start + len(p.tokens))
+        return logits
+
+    def _portions(self, entries) -> list[Portion]:
+        """The step's entries, checked, as portions at their requests' present lengths."""
         vocab = self.model.spec.vocab_size
         portions = []
         seen = set()
@@ -216,10 +229,54 @@ class ModelRunner:
             if low < 0 or high >= vocab:
                 raise ValueError(f"request {request!r}: token id outside the vocabulary of {vocab}")
             portions.append(Portion(request, ids, start, want))
-        self.cache.extend_all([(p.request, p.start + len(p.tokens)) for p in portions])
+        return portions
+
+    def _batch(self, portions: Sequence[Portion]) -> StepBatch:
         tables = {name: [self.cache.table(p.request, name) for p in portions] for name in self.cache.groups}
-        batch = self.builder.build(portions, tables, [self.cache.slot(p.request) for p in portions])
-        logits = self._forward(batch)
+        return self.builder.build(portions, tables, [self.cache.slot(p.request) for p in portions])
+
+    # ---- several greedy decode steps without the host in between ---------
+    def decode_greedy(self, entries: Sequence[tuple[Hashable, int]], steps: int) -> list[list[int]]:
+        """``entries``: (request, its next token), one decoded token each.
+        Runs up to ``steps`` decode steps one after the other, each request's
+        arg-max token becoming its next token on the device, and returns the
+        chosen tokens step by step, ``[steps run][request]``: the same tokens
+        as as many calls of ``step`` with an arg-max each, with one wait for
+        the device instead of one a step.
+
+        The steps after the first replay the graph captured for the shape, so
+        fewer than ``steps`` are run (at least one) where there is none yet,
+        where the contexts would leave the graph's bucket, or where the cache
+        has no pages for all of them."""
+        if not entries:
+            return []
+        portions = self._portions([(request, [token], [0]) for request, token in entries])
+        longest = max(p.start + 1 for p in portions)
+        run = max(1, min(int(steps), self.config.max_model_len - longest + 1))
+        key = None
+        if run > 1:
+            key = self._decode_graph_key(len(portions), longest)
+            if key is None or key not in self._graphs:
+                run = 1
+            else:
+                run = min(run, key[1] - longest + 1)  # the last step's contexts still inside the bucket
+        if run > 1 and not self.cache.can_extend([(p.request, p.start + run) for p in portions]):
+            run = 1
+        self.cache.extend_all([(p.request, p.start + run) for p in portions])
+        batch = self._batch(portions)
+        chosen = torch.empty((run, len(portions)), dtype=torch.int32, device=self.device)
+        for i in range(run):
+            if i > 0:
+                ops.advance_decode(batch, chosen[i - 1])
+            logits = self._forward(batch) if i == 0 else self._replay(key)
+            ops.argmax(logits, out=chosen[i])
         for p in portions:
-            self.cache.commit(p.request, p.start + len(p.tokens))
-        return logits
+            self.cache.commit(p.request, p.start + run)
+        return chosen.cpu().tolist()
+
+    def _replay(self, key) -> torch.Tensor:
+        graph, static_logits = self._graphs[key]
+        self._graphs.move_to_end(key)
+        graph.replay()
+        self.graph_replays += 1
+        return static_logits

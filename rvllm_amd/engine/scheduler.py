@@ -63,6 +63,16 @@ class Request:
     def tokens(self) -> list[int]:
         return self.prompt + self.output
 
+    def tokens_at(self, start: int, count: int) -> list[int]:
+        """``tokens[start : start + count]`` without joining the lists (a step asks every request for its next
+        tokens, and a long request's whole list is long)."""
+        n = len(self.prompt)
+        if start >= n:
+            return self.output[start - n : start - n + count]
+        if start + count <= n:
+            return self.prompt[start : start + count]
+        return self.prompt[start:] + self.output[: start + count - n]
+
     @property
     def total(self) -> int:
         return len(self.prompt) + len(self.output)

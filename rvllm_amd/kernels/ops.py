@@ -575,6 +575,19 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     return out
 
 
+def advance_decode(step, chosen: torch.Tensor) -> None:
+    """A step of decoded tokens becomes the next one on the device: request b's
+    next token is ``chosen[b]``, one position on.  ``step`` is the step's batch
+    (token b belongs to request b); its arrays are changed in place."""
+    n = step.num_requests
+    _need(step.num_tokens == n and step.max_portion == 1, "advance_decode: a step of single decoded tokens expected")
+    _gpu(chosen, step.token_ids, step.positions, step.chunk_start, step.context_len)
+    _i32(chosen, step.token_ids, step.positions, step.chunk_start, step.context_len)
+    _need(chosen.numel() == n, "advance_decode: one chosen token per request expected")
+    _check(library().rv_advance_decode(_stream(), _ptr(chosen), _ptr(step.token_ids), _ptr(step.positions),
+                                       _ptr(step.chunk_start), _ptr(step.context_len), _c_int(n)))
+
+
 def topk_select(logits: torch.Tensor, k: int, inv_temp: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """The k largest logits of every row, times 1/T, with their ids (unordered)."""
     _gpu(logits, inv_temp)

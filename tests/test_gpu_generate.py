@@ -190,6 +190,79 @@ def test_a_graph_dropped_for_room_is_recorded_again(model_dirs, plain_models):
     assert replays == [0, 1, 1, 1, 1] * 3  # the first step of each run of a shape is eager
 
 
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_several_greedy_steps_in_a_row_choose_what_single_steps_choose(model_dirs, name):
+    """``decode_greedy`` hands each request's arg-max token to its next step on the device.  Against a twin runner
+    that takes one step at a time: the same tokens, over page edges, with requests of different lengths; one step
+    only while the shape has no graph yet, and no step past the end of the graph's bucket of contexts."""
+    common = dict(dtype="bfloat16", max_model_len=1100, max_num_seqs=4, max_num_batched_tokens=1100,
+                  max_prefill_chunk=1100, max_cache_tokens=3400, use_graphs=True)
+    one = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(**common)).runner
+    many = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(**common)).runner
+    vocab = one.model.spec.vocab_size
+    prompts = {"a": [(7 * i + 1) % vocab for i in range(10)], "b": [(3 * i + 2) % vocab for i in range(27)],
+               "c": [(5 * i + 3) % vocab for i in range(1000)]}  # c is 19 tokens from the end of the first bucket
+    last = {}
+    for runner in (one, many):
+        for rid, ids in prompts.items():
+            runner.add_request(rid)
+            last[rid] = int(runner.step([(rid, ids, [len(ids) - 1])]).argmax())
+    nxt_one, nxt_many = dict(last), dict(last)
+    taken = []
+    total = 0
+    while total < 40:
+        rows = many.decode_greedy([(rid, nxt_many[rid]) for rid in prompts], 6)
+        taken.append(len(rows))
+        for row in rows:
+            got = one.step([(rid, [nxt_one[rid]], [0]) for rid in prompts]).argmax(dim=1).tolist()
+            assert row == got, f"step {total}"
+            nxt_one = dict(zip(prompts, got))
+            total += 1
+        nxt_many = dict(zip(prompts, rows[-1]))
+        assert {rid: many.length(rid) for rid in prompts} == {rid: one.length(rid) for rid in prompts}
+    # the first call meets a shape without a graph; the contexts reach 1024 after 24 steps: the call before
+    # runs only as far as the bucket goes, the one after starts a new shape
+    assert taken[0] == 1 and max(taken) == 6 and sum(taken[: taken.index(1, 1)]) == 24, taken
+    assert many.graph_replays > one.graph_replays // 2
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_greedy_steps_ahead_change_no_token(model_dirs, name):
+    """Several greedy decode steps from one plan against one plan a step: the same tokens and reasons for requests
+    that end at different lengths, one of them at an end id met on the way, with a request that samples among them
+    (then every step is planned by itself), and with so few pages that requests are set back."""
+    def run(ahead, tight):
+        engine = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(
+            dtype="bfloat16", max_model_len=200, max_num_seqs=4, max_num_batched_tokens=64, max_prefill_chunk=64,
+            max_cache_tokens=160 if tight else 800, greedy_steps_ahead=ahead))
+        vocab = engine.runner.model.spec.vocab_size
+        prompts = [[(11 * i + j) % vocab for i in range(n)] for j, n in enumerate((5, 18, 33, 9))]
+        out = {}
+        for phase, sampled in (("all greedy", False), ("one samples", True)):
+            for j, prompt in enumerate(prompts):
+                params = SamplingParams(0.9, 20, 1.0, seed=3) if sampled and j == 2 else SamplingParams()
+                engine.add_request((phase, j), prompt, params, max_new_tokens=(37, 50, 23, 44)[j],
+                                   eos_ids=run.eos if j == 1 else (), ignore_eos=False)
+            while engine.has_work():
+                for res in engine.step():
+                    out[res.request_id] = (res.tokens, res.finish_reason)
+        return out, engine
+
+    run.eos = ()
+    free, _ = run(1, False)
+    run.eos = (free[("all greedy", 1)][0][29],)  # request 1 will stop at this token, or at its first appearance
+    single, e1 = run(1, False)
+    ahead, e4 = run(4, False)
+    assert single == ahead
+    assert single[("all greedy", 1)][1] == "stop" and len(single[("all greedy", 1)][0]) <= 30
+    assert [single[("all greedy", j)][1] for j in (0, 2, 3)] == ["length"] * 3
+    assert e4.steps == e1.steps  # a step is a step, however many were planned at once
+    assert e1.plans == e1.steps and e4.plans < 0.7 * e4.steps
+    tight_single, t1 = run(1, True)
+    tight_ahead, t4 = run(4, True)
+    assert tight_single == tight_ahead == single
+
+
 def test_eos_and_capacity_reasons(model_dirs):
     engine = LLMEngine.from_model_dir(model_dirs["A"], EngineConfig(dtype="float32", max_model_len=128,
                                                                     max_num_seqs=2, max_cache_tokens=32))

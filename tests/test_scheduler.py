@@ -207,3 +207,12 @@ def test_state_changes_only_after_the_step():
     assert req.state is RequestState.RUNNING and req.computed == 0 and req.output == []
     sched.commit(plan, runner.step(plan))
     assert req.computed == 3 and len(req.output) == 1
+
+
+def test_a_requests_tokens_from_a_place_on():
+    from rvllm_amd.engine.scheduler import Request
+
+    req = Request("r", [1, 2, 3, 4], output=[5, 6, 7])
+    for start in range(7):
+        for count in range(1, 8 - start):
+            assert req.tokens_at(start, count) == req.tokens[start:start + count], (start, count)
