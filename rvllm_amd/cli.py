@@ -52,6 +52,7 @@ USAGE = """usage: rvllm-amd --model DIR [options]
   --dump FILE                    write the generated ids, one request per line         [$RVLLM_GEN_DUMP]
   --random-weights CONFIG.json   no folder: random weights for this configuration (with --weights-seed S)
   --no-graphs                    do not replay decode steps from captured HIP graphs   [$RVLLM_GRAPHS=0]
+  --greedy-steps-ahead N         greedy decode steps that may follow one another without the host (default 4, 1 = off)
   --dry-run                      check the configuration and the arguments, load nothing
 """
 
@@ -90,10 +91,11 @@ def parse(argv: list[str], env: dict) -> dict:
         "random_weights": None, "weights_seed": 0,
         "dry_run": env.get("RVLLM_DRY_RUN", "") not in ("", "0", "false"),
         "graphs": env.get("RVLLM_GRAPHS", "1") not in ("0", "false"),
+        "greedy_steps_ahead": 4,
     }
     ints = {"--max-model-len", "--max-num-seqs", "--max-inflight-requests", "--max-num-batched-tokens",
             "--max-prefill-chunk", "--page-size", "--max-cache-tokens", "--prompt-len", "--max-tokens", "--top-k",
-            "--seed", "--weights-seed"}
+            "--seed", "--weights-seed", "--greedy-steps-ahead"}
     floats = {"--temperature", "--top-p"}
     strings = {"--model", "--dtype", "--prompt-file", "--eos", "--dump", "--random-weights"}
     it = iter(argv)
@@ -177,7 +179,7 @@ def main(argv=None, env=None) -> int:
         cfg = EngineConfig(dtype=o["dtype"], page_size=o["page_size"], max_model_len=o["max_model_len"],
                            max_num_seqs=o["max_num_seqs"], max_num_batched_tokens=o["max_num_batched_tokens"],
                            max_prefill_chunk=o["max_prefill_chunk"], max_cache_tokens=o["max_cache_tokens"],
-                           use_graphs=o["graphs"]).validate()
+                           use_graphs=o["graphs"], greedy_steps_ahead=o["greedy_steps_ahead"]).validate()
         if o["random_weights"]:
             doc = json.loads(Path(o["random_weights"]).read_text())
             arch = architecture_of(doc, o["random_weights"])
