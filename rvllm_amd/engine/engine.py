@@ -107,11 +107,15 @@ class LLMEngine:
         """How many decode steps may follow one another from this plan: more
         than one only if every request in it decodes greedily, none could end
         by its length or the model's on the way, nothing was set back, and no
-        request waits (it would be admitted that much later).  A request that
-        meets an end id on the way stops there; what was run for it after
+        request waits for which there is a place (it would be admitted that
+        much later; with every place taken, the most a waiting request can
+        lose is the few steps by which an end id is noticed late).  A request
+        that meets an end id on the way stops there; what was run for it after
         that is dropped, and costs the others nothing."""
         ahead = self.runner.config.greedy_steps_ahead
-        if ahead <= 1 or self.scheduler.waiting or plan.set_back:
+        if ahead <= 1 or plan.set_back:
+            return 1
+        if self.scheduler.waiting and len(self.scheduler.running) < self.scheduler.max_num_seqs:
             return 1
         for p in plan.portions:
             req = p.request

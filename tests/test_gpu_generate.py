@@ -231,9 +231,9 @@ def test_greedy_steps_ahead_change_no_token(model_dirs, name):
     """Several greedy decode steps from one plan against one plan a step: the same tokens and reasons for requests
     that end at different lengths, one of them at an end id met on the way, with a request that samples among them
     (then every step is planned by itself), and with so few pages that requests are set back."""
-    def run(ahead, tight):
+    def run(ahead, tight, places=4):
         engine = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(
-            dtype="bfloat16", max_model_len=200, max_num_seqs=4, max_num_batched_tokens=64, max_prefill_chunk=64,
+            dtype="bfloat16", max_model_len=200, max_num_seqs=places, max_num_batched_tokens=64, max_prefill_chunk=64,
             max_cache_tokens=160 if tight else 800, greedy_steps_ahead=ahead))
         vocab = engine.runner.model.spec.vocab_size
         prompts = [[(11 * i + j) % vocab for i in range(n)] for j, n in enumerate((5, 18, 33, 9))]
@@ -261,6 +261,11 @@ def test_greedy_steps_ahead_change_no_token(model_dirs, name):
     tight_single, t1 = run(1, True)
     tight_ahead, t4 = run(4, True)
     assert tight_single == tight_ahead == single
+    # two places for four requests: the waiting ones get theirs when a running one ends, and steps follow one
+    # another meanwhile
+    few_single, f1 = run(1, False, places=2)
+    few_ahead, f4 = run(4, False, places=2)
+    assert few_single == few_ahead == single and f4.plans < 0.8 * f4.steps
 
 
 def test_eos_and_capacity_reasons(model_dirs):
