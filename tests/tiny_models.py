@@ -132,8 +132,31 @@ CONFIG_E = {
     "final_logit_softcapping": None,
 }
 
+# The whole model at the sizes of Gemma 3 4B: 34 layers, every sixth one global, the full vocabulary.
+CONFIG_4B = {
+    "architectures": ["Gemma3ForCausalLM"],
+    "num_hidden_layers": 34,
+    "sliding_window_pattern": 6,
+    "hidden_size": 2560,
+    "num_attention_heads": 8,
+    "num_key_value_heads": 4,
+    "head_dim": 256,
+    "intermediate_size": 10240,
+    "vocab_size": 262208,
+    "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 131072,
+    "sliding_window": 1024,
+    "rope_theta": 1000000.0,
+    "rope_local_base_freq": 10000.0,
+    "rope_scaling": {"rope_type": "linear", "factor": 8.0},
+    "query_pre_attn_scalar": 256,
+    "hidden_activation": "gelu_pytorch_tanh",
+    "tie_word_embeddings": True,
+    "final_logit_softcapping": None,
+}
+
 CONFIGS = {"A": (CONFIG_A, 0), "B": (CONFIG_B, 1), "C": (CONFIG_C, 2)}
-LARGER = {"D": (CONFIG_D, 3), "E": (CONFIG_E, 4)}
+LARGER = {"D": (CONFIG_D, 3), "E": (CONFIG_E, 4), "4B": (CONFIG_4B, 5)}
 
 
 def write_model(folder, name: str, dtype=torch.bfloat16, seed=None) -> Path:
