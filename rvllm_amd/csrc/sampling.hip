@@ -10,7 +10,10 @@
 //             (v3/kernels/sample_topk_f32.cu:1-13,68-117)
 #include <math.h>
 
+#include <mutex>
+
 #include "common.h"
+#include "no_alloc.h"
 
 // ---------------------------------------------------------------------------
 // arg-max in two stages, so that a row of 262 208 logits is read by many CUs.
@@ -107,6 +110,63 @@ extern "C" int rv_argmax(hipStream_t stream, const float* logits, int rows, int 
   RV_LAUNCH_CHECK("argmax_partial");
   argmax_final_kernel<<<dim3(rows), dim3(256), 0, stream>>>(ws_val, ws_idx, parts, out);
   RV_LAUNCH_CHECK("argmax_final");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The same arg-max for callers that cannot allocate: the first stage's partial
+// results go to an array that the library holds in device memory.  Each GPU
+// has its own copy of the array at its own address; the name `scratch` is only
+// a stand-in on the host, so the address is asked for once per device and kept.
+// ---------------------------------------------------------------------------
+#define RV_NO_ALLOC_SLOTS (RV_NO_ALLOC_MAX_ROWS * RV_NO_ALLOC_MAX_PARTS)
+static __device__ __align__(256) unsigned char scratch[RV_NO_ALLOC_SLOTS * (sizeof(float) + sizeof(int))];
+
+#define RV_MAX_DEVICES 64
+static void* g_scratch_ptr[RV_MAX_DEVICES];  // the array's address on each device, once asked for
+static std::mutex g_scratch_lock;
+
+// The address of `scratch` on the current device; null (with the error set) when it cannot be had.
+static void* scratch_on_current_device() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= RV_MAX_DEVICES) {
+    rv_fail("argmax_no_alloc: no current device (%s, device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      rv_fail("argmax_no_alloc: the address of the scratch array on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+extern "C" int rv_argmax_no_alloc(hipStream_t stream, const float* logits, int rows, int vocab, long long row_stride,
+                                  int* out) {
+  RV_CHECK(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax_no_alloc: bad sizes rows=%d vocab=%d", rows, vocab);
+  RV_CHECK(logits && out, "argmax_no_alloc: null logits or output");
+  RV_CHECK(rows <= RV_NO_ALLOC_MAX_ROWS, "argmax_no_alloc: %d rows, the scratch array holds %d", rows,
+           RV_NO_ALLOC_MAX_ROWS);
+  if (rows == 0) return 0;
+  const int parts = rv_argmax_parts(vocab);
+  RV_CHECK(parts <= RV_NO_ALLOC_MAX_PARTS, "argmax_no_alloc: %d parts a row, the scratch array holds %d", parts,
+           RV_NO_ALLOC_MAX_PARTS);
+  void* ptr = scratch_on_current_device();
+  if (!ptr) return -1;
+  // Values first, then ids.  Every slot the second stage reads is written by the first, so what an earlier
+  // call left in the array is never seen.
+  float* ws_val = (float*)ptr;
+  int* ws_idx = (int*)((unsigned char*)ptr + RV_NO_ALLOC_SLOTS * sizeof(float));
+  argmax_partial_kernel<<<dim3(parts, rows), dim3(256), 0, stream>>>(logits, vocab, row_stride, parts, ws_val, ws_idx);
+  RV_LAUNCH_CHECK("argmax_partial (no alloc)");
+  argmax_final_kernel<<<dim3(rows), dim3(256), 0, stream>>>(ws_val, ws_idx, parts, out);
+  RV_LAUNCH_CHECK("argmax_final (no alloc)");
   return 0;
 }
 
