@@ -18,7 +18,14 @@ One JSON line goes to standard output.  ``value`` is decoded tokens a second.
 ``roofline`` prices the decode step against 8 TB/s: the bytes it must read
 (every weight it uses once, and the keys and values of the live requests that
 a token may see) over its time.  ``prefill.frac`` prices the prompt's flops
-against 2.5 PFLOP/s (dense bf16 MFMA).
+against 2.5 PFLOP/s (dense bf16 MFMA).  Beside the vendor's peaks stand
+measured ones (``measured_peak``): what a kernel that only reads gets from the
+memory (the engine's own probe kernel over 4 GiB), and what the library's bf16
+product of 8192 x 8192 x 8192 reaches (hipBLASLt through torch.matmul).
+
+The timed decode steps end at the named context: the caches are filled so that
+the last timed step sees exactly ``--context`` tokens, and every step runs
+under the attention plan (and graph) of that context's bucket.
 """
 
 from __future__ import annotations
@@ -98,7 +105,7 @@ def fill_cache(runner, batch: int, context: int, torch):
     for b in range(batch):
         rid = f"bench-{b}"
         runner.add_request(rid)
-        runner.cache.adopt_length(rid, context)
+        runner.cache.adopt_length_for_measurement(rid, context)
         ids.append(rid)
     gen = torch.Generator(device=runner.device)
     gen.manual_seed(1)
@@ -116,7 +123,7 @@ def release_all(runner, ids):
 
 def time_decode(engine_parts, batch: int, context: int, steps: int, warmup: int):
     torch, runner, sampler, SamplingParams, SplitMix64 = engine_parts
-    ids = fill_cache(runner, batch, context - 1, torch)
+    ids = fill_cache(runner, batch, max(1, context - steps - warmup), torch)  # the last timed step sees `context`
     params = [SamplingParams() for _ in ids]
     rngs = [SplitMix64(0) for _ in ids]
     tokens = [(17 * b + 5) % runner.model.spec.vocab_size for b in range(batch)]
@@ -151,7 +158,7 @@ def time_prefill(engine_parts, length: int, repeats: int):
     g = torch.Generator().manual_seed(2)
     prompt = torch.randint(0, vocab, (length,), generator=g).tolist()
     runner.warm_up([length])  # first-use work, and the library's products tuned for this shape
-    best = None
+    times = []
     for i in range(repeats + 1):
         rid = f"prefill-{i}"
         runner.add_request(rid)
@@ -163,8 +170,48 @@ def time_prefill(engine_parts, length: int, repeats: int):
         dt = time.perf_counter() - t0
         runner.release(rid)
         if i > 0:  # the first run warms up
-            best = dt if best is None else min(best, dt)
-    return best
+            times.append(dt)
+    return sum(times) / len(times), min(times)
+
+
+def measure_peaks(torch, device, short: str) -> dict:
+    """What this machine gives a kernel that only reads, and the library's best product: the peaks one can
+    reach, beside the vendor's.  Both take the best of several runs."""
+    from rvllm_amd.kernels import ops
+
+    out = {}
+    buf = torch.empty(4 << 30, dtype=torch.uint8, device=device)  # far more than the caches hold
+    buf.zero_()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = None
+    for i in range(6):
+        start.record()
+        ops.probe_read(buf, blocks=4096)
+        stop.record()
+        stop.synchronize()
+        ms = start.elapsed_time(stop)
+        if i > 0:
+            best = ms if best is None else min(best, ms)
+    out["hbm_read_GBs"] = round(buf.numel() / (best * 1e-3) / 1e9, 1)
+    del buf
+    if short == "bf16":
+        n = 8192
+        a = torch.randn((n, n), device=device, dtype=torch.bfloat16)
+        b = torch.randn((n, n), device=device, dtype=torch.bfloat16)
+        c = torch.empty((n, n), device=device, dtype=torch.bfloat16)
+        best = None
+        for i in range(6):
+            start.record()
+            torch.matmul(a, b.t(), out=c)
+            stop.record()
+            stop.synchronize()
+            ms = start.elapsed_time(stop)
+            if i > 0:
+                best = ms if best is None else min(best, ms)
+        out["gemm_bf16_TFLOPs"] = round(2 * n ** 3 / (best * 1e-3) / 1e12, 1)
+        del a, b, c
+    torch.cuda.empty_cache()
+    return out
 
 
 # The engine workloads of the larger configurations: requests through the scheduler, prompts cut into portions
@@ -203,6 +250,31 @@ def run_workload(name: str, requests, layers) -> int:
     log(f"building the {name}-sized model ({cfg.num_hidden_layers} layers) with random weights")
     engine = LLMEngine.from_random(cfg, 0, engine_cfg)
     engine.runner.warm_up([portion])
+
+    # What every step of the model must at least do, from the plans the scheduler commits: the bytes it reads
+    # (all weights once, the keys and values its tokens may see) and its flops (products, attention, head).
+    weight_bytes, layer_flops_per_token, head_flops_per_row = model_numbers(cfg, 2)
+    kv_token_bytes = 2 * cfg.kv_size * 2
+    tally = {"steps": 0, "bytes": 0, "flops": 0, "ideal_s": 0.0}
+    commit = engine.scheduler.commit
+
+    def counting_commit(plan, next_tokens):
+        step_bytes, step_flops = weight_bytes, 0
+        for p in plan.portions:
+            for l in range(cfg.num_hidden_layers):
+                seen = p.start + p.count
+                if cfg.is_sliding(l):
+                    seen = min(seen, cfg.sliding_window - 1 + p.count)
+                step_bytes += seen * kv_token_bytes
+            step_flops += p.count * layer_flops_per_token + attention_flops(cfg, p.start, p.count)
+            step_flops += head_flops_per_row if p.wants_token else 0
+        tally["steps"] += 1
+        tally["bytes"] += step_bytes
+        tally["flops"] += step_flops
+        tally["ideal_s"] += max(step_bytes / (PEAK_HBM_GBS * 1e9), step_flops / PEAK_FLOPS["bf16"])
+        return commit(plan, next_tokens)
+
+    engine.scheduler.commit = counting_commit
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     results = engine.generate(prompts, [SamplingParams() for _ in prompts], new, (), True)
@@ -213,6 +285,13 @@ def run_workload(name: str, requests, layers) -> int:
         "metric": f"tokens/s through the engine, {name}-sized workload", "value": round((sum(lengths) + made) / sec, 1),
         "unit": "tok/s", "n_gpus": 1, "seconds": round(sec, 2), "higher_is_better": True, "dtype": "bf16",
         "data": "synthetic: random weights, uniform token ids, greedy",
+        # every step priced at the slower of its bytes at 8 TB/s and its flops at 2.5 PFLOP/s; `frac` is the
+        # sum of these times over the run's time
+        "roofline": {"bound": "per step: max(hbm, mfma)", "steps": tally["steps"],
+                     "bytes_TB": round(tally["bytes"] / 1e12, 3), "flops_PFLOP": round(tally["flops"] / 1e15, 3),
+                     "ideal_seconds": round(tally["ideal_s"], 3), "frac": round(tally["ideal_s"] / sec, 4),
+                     "achieved_GBs": round(tally["bytes"] / sec / 1e9, 1),
+                     "achieved_TFLOPs": round(tally["flops"] / sec / 1e12, 1)},
         "config": {"model": f"gemma3-{name}-sized dense decoder", "requests": n_req, "prompt_tokens": sum(lengths),
                    "new_tokens": made, "portion": portion, "layers": cfg.num_hidden_layers,
                    "layers_of_named_config": full_layers, "hidden_size": cfg.hidden_size, "head_dim": cfg.head_dim,
@@ -233,6 +312,7 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-probes", action="store_true", help="skip the measured peaks (read rate, library product)")
     ap.add_argument("--graphs", type=int, default=1, help="replay decode steps from captured HIP graphs (0 = off)")
     ap.add_argument("--steps-ahead", type=int, default=None,
                     help="greedy decode steps that follow one another without the host (1 = off; default: the engine's)")
@@ -241,7 +321,7 @@ def main() -> int:
     ap.add_argument("--requests", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
-        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine", flush=True)
         return 2
     if args.workload:
         return run_workload(args.workload, args.requests, args.layers if args.layers != FULL_LAYERS else 0)
@@ -281,12 +361,17 @@ def main() -> int:
         log(f"decode batch {batch}: {sec * 1e3:.3f} ms/step, {batch / sec:.1f} tok/s")
         return sec
 
+    peaks = {} if args.no_probes else measure_peaks(torch, runner.device, short)
+    if peaks:
+        log(f"measured peaks: {peaks}")
     sec = decode_point(args.batch, args.steps, args.warmup)
     value = args.batch / sec
-    step_bytes = weight_bytes + args.batch * kv_bytes_per_request(cfg, args.context, elem)
+    # the timed steps see context - steps + 1 .. context tokens: priced at their mean
+    mean_context = max(1, args.context - (args.steps - 1) // 2)
+    step_bytes = weight_bytes + args.batch * kv_bytes_per_request(cfg, mean_context, elem)
     achieved = step_bytes / sec / 1e9
     result = {
-        "metric": "decode tok/s at batch 8, context 8192 (Gemma-3-4B sizes)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Gemma-3-4B sizes)",
         "value": round(value, 2),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -320,13 +405,19 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
+    if "hbm_read_GBs" in peaks:
+        result["roofline"]["measured_peak"] = peaks["hbm_read_GBs"]
+        result["roofline"]["frac_of_measured"] = round(achieved / peaks["hbm_read_GBs"], 4)
     if not args.no_prefill:
         T = args.prefill_tokens
-        psec = time_prefill(parts, T, repeats=5)
+        psec, pmin = time_prefill(parts, T, repeats=5)
         flops = T * layer_flops_per_token + attention_flops(cfg, 0, T) + head_flops_per_row
         result["prefill"] = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
-                             "frac": round(flops / psec / PEAK_FLOPS[short], 4)}
-        log(f"prefill {T} tokens: {psec * 1e3:.2f} ms, {T / psec:.0f} tok/s")
+                             "frac": round(flops / psec / PEAK_FLOPS[short], 4), "ms_min": round(pmin * 1e3, 3)}
+        if "gemm_bf16_TFLOPs" in peaks:
+            result["prefill"]["measured_peak_TFLOPs"] = peaks["gemm_bf16_TFLOPs"]
+            result["prefill"]["frac_of_measured"] = round(flops / psec / (peaks["gemm_bf16_TFLOPs"] * 1e12), 4)
+        log(f"prefill {T} tokens: {psec * 1e3:.2f} ms mean ({pmin * 1e3:.2f} min), {T / psec:.0f} tok/s")
     if not args.no_points:
         points = {}
         for b in (1, 64):

@@ -39,6 +39,17 @@ class RequestCache:
     tables: dict = dataclasses.field(default_factory=dict)  # group -> BlockTable
 
 
+def window_pages_bound(window: int, page_size: int, max_step_tokens: int) -> int:
+    """The most pages a request ever holds in a group whose layers see a window
+    of ``window`` keys, when a step brings it at most ``max_step_tokens``
+    tokens: the window behind the step's first token, the step's tokens, and
+    one more page because both ends may lie inside a page.  This is what a ring
+    of ``window`` slots per request would reserve, in pages that return to the
+    pool as the window passes them (the reference sizes its sliding layers as
+    ceil(window / block) blocks: v3/crates/rvllm-runtime/src/gemma4_bring_up.rs:3532-3563)."""
+    return -(-(window - 1 + max_step_tokens) // page_size) + 1
+
+
 class PageGroup:
     def __init__(self, name: str, window: Optional[int], page_size: int, num_pages: int):
         self.name = name
@@ -209,7 +220,7 @@ class CacheManager:
                 if n:
                     rc.tables[name].extend(self.groups[name].pool.take(rc.request, n))
 
-    def adopt_length(self, request: Hashable, length: int) -> None:
+    def adopt_length_for_measurement(self, request: Hashable, length: int) -> None:
         """Make a fresh request hold ``length`` tokens without running them:
         it gets exactly the pages a request of that length holds (none behind
         a window).  For measurements on a cache filled by hand."""

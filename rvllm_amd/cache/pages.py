@@ -39,6 +39,11 @@ class PagePool:
         self.num_pages = num_pages
         self._free = list(range(num_pages - 1, -1, -1))  # pop() gives page 0 first
         self._owner: dict[int, Hashable] = {}
+        self._held: dict[Hashable, int] = {}  # pages each owner holds now
+        self.most_held_by_one = 0  # the most pages any one owner has held at a time
+        # With ``keep_history`` every page remembers its owners in order (tests ask whether pages changed hands).
+        self.keep_history = False
+        self.history: dict[int, list[Hashable]] = {}
 
     @property
     def free_count(self) -> int:
@@ -52,15 +57,33 @@ class PagePool:
             if p in self._owner:
                 raise CacheBookkeepingError(f"page {p} of {self.name!r} handed out while owned by {self._owner[p]!r}")
             self._owner[p] = owner
+            if self.keep_history:
+                self.history.setdefault(p, []).append(owner)
+        if count:
+            held = self._held.get(owner, 0) + count
+            self._held[owner] = held
+            if held > self.most_held_by_one:
+                self.most_held_by_one = held
         return pages
 
     def give_back(self, owner: Hashable, pages) -> None:
+        count = 0
         for p in pages:
             if self._owner.get(p, _NOBODY) != owner:
                 raise CacheBookkeepingError(
                     f"page {p} of {self.name!r} given back by {owner!r} but owned by {self._owner.get(p, 'nobody')!r}")
             del self._owner[p]
             self._free.append(p)
+            count += 1
+        if count:
+            left = self._held[owner] - count
+            if left:
+                self._held[owner] = left
+            else:
+                del self._held[owner]
+
+    def held_by(self, owner: Hashable) -> int:
+        return self._held.get(owner, 0)
 
     def owner_of(self, page: int) -> Optional[Hashable]:
         return self._owner.get(page)
@@ -74,6 +97,8 @@ class PagePool:
             raise CacheBookkeepingError(f"{self.name!r}: a page is free and owned")
         if len(free) + len(self._owner) != self.num_pages:
             raise CacheBookkeepingError(f"{self.name!r}: {self.num_pages - len(free) - len(self._owner)} page(s) lost")
+        if sum(self._held.values()) != len(self._owner):
+            raise CacheBookkeepingError(f"{self.name!r}: the owners' counts do not add up to the pages owned")
 
 
 _NOBODY = object()

@@ -33,7 +33,7 @@ class GenerationResult:
     request_id: Hashable
     prompt: list[int]
     tokens: list[int]
-    finish_reason: str  # "stop" (an end-of-sequence id), "length", or "capacity"
+    finish_reason: str  # "stop" (an end-of-sequence id), "length", "capacity", or "error" (its step failed)
     set_backs: int = 0
 
 
@@ -94,10 +94,18 @@ class LLMEngine:
         ahead = self._greedy_steps_ahead(plan)
         if ahead > 1:
             return results + self._decode_ahead(plan, ahead)
-        logits = self.runner.step(entries)
-        self.steps += 1
-        self.tokens_run += plan.num_tokens
-        chosen = self.sampler.sample(logits, [r.params for r in wanting], [r.rng for r in wanting])
+        try:
+            logits = self.runner.step(entries, starts=[p.start for p in plan.portions])
+            self.steps += 1
+            self.tokens_run += plan.num_tokens
+            chosen = self.sampler.sample(logits, [r.params for r in wanting], [r.rng for r in wanting])
+        except Exception:
+            # The cache may hold this step's tokens while the requests do not count them (the sampler refuses
+            # logits that are not finite, for one): the plan's requests end here, so that nothing is run twice
+            # or a portion further on, and the others go on.
+            for p in plan.portions:
+                self.scheduler.abort(p.request, "error")
+            raise
         next_tokens = {r.id: t for r, t in zip(wanting, chosen)}
         finished = self.scheduler.commit(plan, next_tokens)
         return results + [self._result(r) for r in finished]

@@ -12,26 +12,22 @@ from __future__ import annotations
 import collections
 import dataclasses
 import os
+import warnings
 from typing import Hashable, Optional, Sequence
 
 import numpy as np
 import torch
 
-from ..cache.manager import CacheManager, group_name
+from ..cache.manager import CacheManager, group_name, window_pages_bound
 from ..cache.storage import CacheStorage
 from ..config.engine_config import EngineConfig
 from ..kernels import ops
 from ..models.model import DecoderModel
 from ..models.registry import Architecture, get_architecture, load_config
 from ..parts.base import KVNeed
-from ..weights.loader import detect_prefix, load_tensors, open_model_files, tensor_names
+from ..weights.loader import load_tensors, open_model_files, tensor_names
 from ..weights.random_init import random_tensors
 from .batch import BatchBuilder, Portion, StepBatch
-
-# Tensors of a multimodal checkpoint that the text decoder leaves alone.
-IGNORED_TENSOR_PREFIXES = ("vision_tower.", "model.vision_tower.", "multi_modal_projector.",
-                           "model.multi_modal_projector.")
-
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, engine_config: EngineConfig):
@@ -40,6 +36,12 @@ class ModelRunner:
         self.config = engine_config.validate()
         self.device = model.device
         self.dtype = model.dtype
+        if self.config.max_model_len > model.spec.max_position:
+            # the reference caps a request the same way: prompt + new tokens <= min(cache, max_position_embeddings)
+            # (v3/crates/rvllm-runtime/src/gemma4_bring_up.rs:271-294)
+            warnings.warn(f"max_model_len {self.config.max_model_len} is more than the model's "
+                          f"{model.spec.max_position} positions; requests are held to {model.spec.max_position}")
+            self.config = dataclasses.replace(self.config, max_model_len=model.spec.max_position)
         cfg = self.config
         ps = cfg.page_size
         needs = model.cache_needs()
@@ -51,9 +53,7 @@ class ModelRunner:
                 if need.window is None:
                     num_pages[name] = full_pages
                 else:
-                    # A request holds at most the window behind its portion, the
-                    # portion, and the partly filled pages at both ends.
-                    per_request = -(-(need.window - 1 + cfg.max_num_batched_tokens) // ps) + 1
+                    per_request = window_pages_bound(need.window, ps, cfg.max_num_batched_tokens)
                     num_pages[name] = min(full_pages, cfg.max_num_seqs * per_request)
         self.cache = CacheManager(needs, ps, num_pages, cfg.max_num_seqs)
         self.storage = CacheStorage(self.cache, self.device, self.dtype)
@@ -67,7 +67,7 @@ class ModelRunner:
 
     # ---- decode steps from captured graphs -------------------------------
     GRAPH_CONTEXT_BUCKET = 1024
-    GRAPH_MAX_REQUESTS = 64  # beyond this the products go to the library, which stays out of graphs
+    GRAPH_MAX_REQUESTS = ops.SKINNY_MAX_ROWS  # beyond this the products go to the library, which stays out of graphs
     GRAPH_MAX_KEPT = 128     # shapes whose graphs are kept; the one unused for longest goes first
 
     def _graph_key(self, batch: StepBatch):
@@ -86,6 +86,8 @@ class ModelRunner:
     def _decode_graph_key(self, num_requests: int, max_context: int):
         """The key for a step of ``num_requests`` decoded tokens, all wanted, at contexts up to ``max_context``."""
         if not (self.config.use_graphs and self.dtype == torch.bfloat16) or num_requests > self.GRAPH_MAX_REQUESTS:
+            return None
+        if not self.model.capturable:  # a part waits for the device or launches by its data
             return None
         bucket = -(-max_context // self.GRAPH_CONTEXT_BUCKET) * self.GRAPH_CONTEXT_BUCKET
         return num_requests, bucket
@@ -125,10 +127,10 @@ class ModelRunner:
         arch, config = load_config(model_dir)
         files = open_model_files(model_dir)
         try:
-            prefix = detect_prefix(tensor_names(files))
-            model = DecoderModel(arch.build_spec(config, prefix))
+            # where the tensors lie in this checkpoint is the architecture's knowledge
+            model = DecoderModel(arch.build_spec(config, **arch.locate_tensors(tensor_names(files))))
             tensors = load_tensors(files, model.param_specs(), engine_config.torch_dtype, source=str(model_dir),
-                                   ignore=IGNORED_TENSOR_PREFIXES)
+                                   ignore=arch.ignored_prefixes)
             model.bind(tensors, engine_config.device, engine_config.torch_dtype)
         finally:
             for f in files:
@@ -192,17 +194,29 @@ class ModelRunner:
         return self.cache.length(request)
 
     # ---- the step ------------------------------------------------------
-    def step(self, entries: Sequence[tuple[Hashable, Sequence[int], Sequence[int]]]) -> torch.Tensor:
+    def step(self, entries: Sequence[tuple[Hashable, Sequence[int], Sequence[int]]],
+             starts: Optional[Sequence[int]] = None) -> torch.Tensor:
         """``entries``: (request, next tokens, wanted places among them).
 
         Runs only these tokens, as one batch, from the cache that earlier
         steps left; returns float32 logits ``[number of wanted places, vocab]``
         in the order of the entries and of their wanted places.  Raises
         ``OutOfPages`` before anything ran if the cache cannot hold the
-        tokens."""
+        tokens.  The tokens of a request go where its cache ends; a caller
+        that keeps its own count gives it as ``starts`` and gets an error,
+        before anything ran, if the two disagree.
+
+        The logits of a decode step that was replayed from a captured graph
+        lie in that graph's own output buffer: they are valid until the next
+        step of the same shape, so a caller that keeps them longer copies them."""
         if not entries:
             return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32, device=self.device)
         portions = self._portions(entries)
+        if starts is not None:
+            for p, start in zip(portions, starts):
+                if p.start != int(start):
+                    raise ValueError(f"request {p.request!r}: the caller places its tokens at {start}, "
+                                     f"its cache ends at {p.start}")
         self.cache.extend_all([(p.request, p.start + len(p.tokens)) for p in portions])
         logits = self._forward(self._batch(portions))
         for p in portions:

@@ -230,6 +230,14 @@ class Scheduler:
         req.finish_reason = reason
         self.known.pop(req.id, None)
 
+    def abort(self, req: Request, reason: str = "abort") -> None:
+        """Ends a request wherever it stands and gives back what it holds."""
+        if req.state is RequestState.FINISHED:
+            return
+        if req in self.waiting:
+            self.waiting.remove(req)
+        self._finish(req, reason)
+
     # ---- after the step ----------------------------------------------------
     def commit(self, plan: StepPlan, next_tokens: dict) -> list[Request]:
         """The planned step has run.  ``next_tokens[request id]`` is the token

@@ -34,6 +34,7 @@ def parse_args(argv=None) -> argparse.Namespace:
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens that live requests hold at any time (each rounded up to a multiple of 64); "
                         "the cache pool is made for this many")
+    p.add_argument("--max-live", type=int, default=4, help="most requests that are live at a time (default 4)")
     p.add_argument("--page-size", type=int, default=None, help="tokens per cache page (default: the engine's)")
     p.add_argument("--device", default="cuda:0")
     return p.parse_args(argv)
@@ -48,7 +49,7 @@ def main(argv=None) -> int:
     from ..config.engine_config import EngineConfig
     from .runner import ModelRunner
 
-    max_live = 4
+    max_live = int(args.max_live)
     cfg = EngineConfig(dtype=args.dtype, device=args.device)
     if args.page_size is not None:
         cfg.page_size = args.page_size
@@ -73,6 +74,9 @@ def main(argv=None) -> int:
         for e in rec.get("entries", []):
             rid = e["id"]
             if not runner.cache.has_request(rid):
+                if len(runner.cache.requests) >= max_live:
+                    raise SystemExit(f"trace_run: step {step} starts request {rid!r} while {max_live} are live; "
+                                     f"end one first or raise --max-live")
                 runner.add_request(rid)
             entries.append((rid, e["tokens"], e.get("want", [])))
         logits = runner.step(entries)

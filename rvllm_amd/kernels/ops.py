@@ -653,6 +653,17 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
 SKINNY_MAX_ROWS = 64
 
 
+def probe_read(data: torch.Tensor, blocks: int = 2048) -> torch.Tensor:
+    """Reads ``data`` once with a kernel that does nothing else (a measurement of the memory's read rate);
+    returns 64 words folded from what was read."""
+    _gpu(data)
+    nbytes = data.numel() * data.element_size()
+    _need(nbytes % 16 == 0 and data.data_ptr() % 16 == 0, "probe_read: 16-byte aligned data of a multiple of 16 bytes")
+    out = torch.zeros(64, dtype=torch.int32, device=data.device)
+    _check(library().rv_probe_read(_stream(), _ptr(data), _c_ll(nbytes), _ptr(out), _c_int(blocks)))
+    return out
+
+
 def gemm_bf16_gate_up(x: torch.Tensor, w_fours: torch.Tensor, activation: str):
     """act(x @ gate^T) * (x @ up^T) in one kernel, for a bf16 ``x`` of at most 64 rows and ``w_fours`` =
     ``rows_in_fours(gate, up)``: the product applies the activation where it holds the sums, which saves a kernel

@@ -25,7 +25,30 @@ from ..parts.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 from .registry import Architecture, register_architecture
 
 
-def build_spec(cfg: Gemma3Config, prefix: str = "model") -> ModelSpec:
+# Prefixes under which a checkpoint may keep the text decoder
+# (v3/crates/rvllm-loader/src/gemma4_arch.rs:624-658), told apart by where the embedding table lies.
+TENSOR_PREFIXES = ("model.language_model", "language_model.model", "language_model", "model")
+# Tensors of a multimodal checkpoint that the text decoder leaves alone.
+IGNORED_TENSOR_PREFIXES = ("vision_tower.", "model.vision_tower.", "multi_modal_projector.",
+                           "model.multi_modal_projector.")
+
+
+def locate_tensors(names) -> dict:
+    """Where a checkpoint keeps the decoder: the prefix of its layers, and the
+    name of an untied head.  The reference looks the head up as plain
+    ``lm_head.weight`` (v3/crates/rvllm-loader/src/gemma4_load.rs:431-436);
+    checkpoints that nest the decoder keep the head beside it
+    (``language_model.lm_head.weight``), so the name under the prefix's own
+    first parts is tried too."""
+    names = set(names)
+    prefix = next((p for p in TENSOR_PREFIXES if f"{p}.embed_tokens.weight" in names), "model")
+    parts = prefix.split(".")
+    candidates = ["lm_head.weight"] + [".".join(parts[:n]) + ".lm_head.weight" for n in range(len(parts), 0, -1)]
+    head = next((c for c in candidates if c in names), "lm_head.weight")
+    return {"prefix": prefix, "head_weight": head}
+
+
+def build_spec(cfg: Gemma3Config, prefix: str = "model", head_weight: str = "lm_head.weight") -> ModelSpec:
     norm = PartSpec("rmsnorm", {"eps": cfg.rms_norm_eps, "unit_offset": True})
     qk_norm = {"eps": cfg.rms_norm_eps, "unit_offset": True}
     scale = cfg.query_pre_attn_scalar ** -0.5
@@ -57,7 +80,8 @@ def build_spec(cfg: Gemma3Config, prefix: str = "model") -> ModelSpec:
         layers=tuple(layers),
         schedule=tuple(ScheduleEntry(l) for l in range(cfg.num_hidden_layers)),
         final_norm=norm,
-        head=PartSpec("lm_head", {"tied": cfg.tie_word_embeddings, "softcap": cfg.final_logit_softcapping}),
+        head=PartSpec("lm_head", {"tied": cfg.tie_word_embeddings, "softcap": cfg.final_logit_softcapping,
+                                  "weight_name": head_weight}),
         prefix=prefix,
     )
 
@@ -72,4 +96,6 @@ for _name in NAMES:
         read_config=Gemma3Config.from_dict,
         build_spec=build_spec,
         write_config=Gemma3Config.to_dict,
+        locate_tensors=locate_tensors,
+        ignored_prefixes=IGNORED_TENSOR_PREFIXES,
     ))

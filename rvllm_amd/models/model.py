@@ -12,9 +12,9 @@ from typing import Optional
 
 import torch
 
-from ..parts import embedding as _embedding
-from ..parts.base import KVNeed, ParamSpec, StateNeed
-from ..parts.registry import BLOCKS, NORMS
+from ..parts import embedding as _embedding  # noqa: F401  (registers the embedding and the head)
+from ..parts.base import ParamSpec
+from ..parts.registry import BLOCKS, EMBEDDINGS, HEADS, NORMS
 from ..parts.spec import ModelSpec
 
 
@@ -22,10 +22,10 @@ class DecoderModel:
     def __init__(self, spec: ModelSpec):
         self.spec = spec
         H, V = spec.hidden_size, spec.vocab_size
-        self.embedding = _embedding.ScaledEmbedding(spec.embedding, hidden_size=H, vocab_size=V)
+        self.embedding = EMBEDDINGS.build(spec.embedding, hidden_size=H, vocab_size=V)
         self.blocks = [BLOCKS.build(layer.block, layer=layer, hidden_size=H) for layer in spec.layers]
-        self.final_norm = NORMS.build(spec.final_norm, width=H, name="norm")
-        self.head = _embedding.LMHead(spec.head, hidden_size=H, vocab_size=V, embedding=self.embedding)
+        self.final_norm = NORMS.build(spec.final_norm, width=H, name=spec.final_norm_name)
+        self.head = HEADS.build(spec.head, hidden_size=H, vocab_size=V, embedding=self.embedding)
         self.device: Optional[torch.device] = None
         self.dtype: Optional[torch.dtype] = None
 
@@ -51,6 +51,11 @@ class DecoderModel:
         self.final_norm.bind(tensors, self.spec.prefix, self.device, dtype)
         self.head.bind(tensors, self.spec.prefix, self.device, dtype)
 
+    @property
+    def capturable(self) -> bool:
+        """Whether a step of this model may be recorded into a HIP graph: only if every part may."""
+        return all(part.capturable for part in (self.embedding, *self.blocks, self.final_norm, self.head))
+
     # ---- cache needs ---------------------------------------------------
     def cache_needs(self) -> list:
         """For every layer what its mixer keeps between steps (or None for a
@@ -64,7 +69,7 @@ class DecoderModel:
 
         ``caches[i]`` is the cache view of layer i."""
         x = torch.empty((step.num_tokens, self.spec.hidden_size), dtype=self.dtype, device=self.device)
-        self.embedding.forward(step.token_ids, x)
+        self.embedding.forward(step, x)
         schedule = self.spec.schedule
         entered = None
         for i, entry in enumerate(schedule):

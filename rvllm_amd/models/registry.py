@@ -2,8 +2,8 @@
 
 config.json's ``architectures[0]`` picks the entry, as in the reference
 (v3/crates/rvllm-core/src/config/model.rs:14-36,71-80).  An entry knows how to
-read its configuration and how to turn it into a ``ModelSpec``; everything
-else is shared.
+read its configuration, how its checkpoints name their tensors, and how to
+turn both into a ``ModelSpec``; everything else is shared.
 """
 
 from __future__ import annotations
@@ -12,7 +12,7 @@ import dataclasses
 import json
 import os
 from pathlib import Path
-from typing import Any, Callable
+from typing import Any, Callable, Iterable
 
 from ..config.errors import ConfigError, UnknownArchitectureError
 from ..parts.spec import ModelSpec
@@ -20,12 +20,25 @@ from ..parts.spec import ModelSpec
 MAX_CONFIG_BYTES = 4 << 20  # v3/crates/rvllm-core/src/config/model.rs:11
 
 
+def _names_as_written(names: Iterable[str]) -> dict:
+    return {}
+
+
 @dataclasses.dataclass(frozen=True)
 class Architecture:
+    """``locate_tensors`` looks at the names a checkpoint holds and returns the
+    keyword arguments for ``build_spec`` that say where this architecture's
+    tensors lie in it (a prefix, the name of an untied head, ...);
+    ``ignored_prefixes`` are name prefixes of tensors such a checkpoint may hold
+    beside the model's (the other towers of a multimodal one).  The loader and
+    the runner know no architecture's names: they ask here."""
+
     name: str
     read_config: Callable[[dict, str], Any]  # (config.json document, source) -> typed configuration
-    build_spec: Callable[..., ModelSpec]  # (typed configuration, tensor-name prefix="model") -> model description
+    build_spec: Callable[..., ModelSpec]  # (typed configuration, **locate_tensors(names)) -> model description
     write_config: Callable[[Any], dict]  # typed configuration -> config.json document
+    locate_tensors: Callable[[Iterable[str]], dict] = _names_as_written
+    ignored_prefixes: tuple[str, ...] = ()
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}

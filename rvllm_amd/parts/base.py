@@ -35,7 +35,15 @@ class ParamSpec:
 
 
 class Part:
-    """Base of every part."""
+    """Base of every part.
+
+    ``capturable`` says whether the part's ``forward`` may be recorded into a
+    HIP graph and replayed: it must launch the same kernels with the same
+    grids and addresses whatever the data, never wait for the device and never
+    read a result on the host.  A part that does any of that sets it to False,
+    and steps of a model that holds such a part are never taken from a graph."""
+
+    capturable: bool = True
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
         return []
@@ -150,6 +158,24 @@ class PositionEncoding(Part):
         return None
 
 
+class Embedding(Part):
+    """What enters the first layer: ``forward`` fills ``out[tokens, hidden]``
+    from the step (its token ids, and its positions if the part adds learned
+    ones)."""
+
+    def forward(self, step: "StepBatch", out: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Logits from the normed rows: ``forward(x[rows, hidden])`` returns 32-bit
+    ``[rows, vocab]``.  A head is built with the model's embedding in hand
+    (``embedding=``), so that it can share its table."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Mixer(Part):
     """Mixes information between the tokens of a request.  ``forward`` returns
     ``[tokens, hidden]``: a tensor, or ``ops.SlicedSums`` when its last product
@@ -181,6 +207,15 @@ class Block(Part):
 
     mixer: Mixer
     feed_forward: FeedForward
+
+    def parts(self) -> Sequence[Part]:
+        """Every part the block holds (the model asks each whether it can be
+        recorded into a graph)."""
+        return (self.mixer, self.feed_forward)
+
+    @property
+    def capturable(self) -> bool:
+        return all(part.capturable for part in self.parts())
 
     def entry_norm(self) -> Optional[Norm]:
         return None

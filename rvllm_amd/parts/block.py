@@ -35,15 +35,15 @@ class SandwichBlock(Block):
         self.norm_in, self.norm_post_mixer, self.norm_pre_ff, self.norm_post_ff = (
             NORMS.build(layer.norm, width=hidden_size, name=name) for name in self.NORM_NAMES)
 
-    def _parts(self):
+    def parts(self):
         return (self.mixer, self.feed_forward, self.norm_in, self.norm_post_mixer, self.norm_pre_ff,
                 self.norm_post_ff)
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
-        return [s for part in self._parts() for s in part.param_specs(prefix)]
+        return [s for part in self.parts() for s in part.param_specs(prefix)]
 
     def bind(self, tensors, prefix, device, dtype) -> None:
-        for part in self._parts():
+        for part in self.parts():
             part.bind(tensors, prefix, device, dtype)
 
     def entry_norm(self) -> Optional[Norm]:

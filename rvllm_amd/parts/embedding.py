@@ -18,51 +18,68 @@ from typing import Optional
 import torch
 
 from ..kernels import ops
-from .base import ParamSpec, Part
+from .base import Embedding, Head, ParamSpec
 from .linear import linear
+from .registry import EMBEDDINGS, HEADS
 from .spec import PartSpec
 
 
-class ScaledEmbedding(Part):
+class ScaledEmbedding(Embedding):
+    """Parameters: ``scale`` (1 if absent) and ``name``, the table's name under
+    the model's prefix (``embed_tokens`` if absent)."""
+
     def __init__(self, spec: PartSpec, *, hidden_size: int, vocab_size: int):
         self.hidden_size = hidden_size
         self.vocab_size = vocab_size
         self.scale = float(spec.get("scale", 1.0))
+        self.name = str(spec.get("name", "embed_tokens"))
         self.table: Optional[torch.Tensor] = None
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
-        return [ParamSpec(f"{prefix}.embed_tokens.weight", (self.vocab_size, self.hidden_size))]
+        return [ParamSpec(f"{prefix}.{self.name}.weight", (self.vocab_size, self.hidden_size))]
 
     def bind(self, tensors, prefix, device, dtype) -> None:
-        self.table = tensors[f"{prefix}.embed_tokens.weight"].to(device=device, dtype=dtype).contiguous()
+        self.table = tensors[f"{prefix}.{self.name}.weight"].to(device=device, dtype=dtype).contiguous()
 
-    def forward(self, token_ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        return ops.embed_gather(self.table, token_ids, self.scale, out)
+    def forward(self, step, out: torch.Tensor) -> torch.Tensor:
+        return ops.embed_gather(self.table, step.token_ids, self.scale, out)
 
 
-class LMHead(Part):
-    def __init__(self, spec: PartSpec, *, hidden_size: int, vocab_size: int, embedding: ScaledEmbedding):
+class LMHead(Head):
+    """Parameters: ``tied`` (the head reads the embedding's table, which must
+    then have a ``table``), ``softcap`` (None: off) and ``weight_name``, the
+    whole name of an untied head's matrix (``lm_head.weight`` if absent: the
+    reference looks it up under no prefix, gemma4_load.rs:431-436)."""
+
+    def __init__(self, spec: PartSpec, *, hidden_size: int, vocab_size: int, embedding):
         self.hidden_size = hidden_size
         self.vocab_size = vocab_size
         self.tied = bool(spec.get("tied", True))
         cap = spec.get("softcap")
         self.softcap = None if cap is None else float(cap)
+        self.weight_name = str(spec.get("weight_name", "lm_head.weight"))
         self.embedding = embedding
         self.weight: Optional[torch.Tensor] = None
+        if self.tied and not hasattr(embedding, "table"):
+            raise ValueError("a tied head needs an embedding that keeps its table as `table`")
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
         if self.tied:
             return []
-        return [ParamSpec("lm_head.weight", (self.vocab_size, self.hidden_size))]
+        return [ParamSpec(self.weight_name, (self.vocab_size, self.hidden_size))]
 
     def bind(self, tensors, prefix, device, dtype) -> None:
         if self.tied:
             self.weight = self.embedding.table
         else:
-            self.weight = tensors["lm_head.weight"].to(device=device, dtype=dtype).contiguous()
+            self.weight = tensors[self.weight_name].to(device=device, dtype=dtype).contiguous()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = linear(x, self.weight, out_dtype=torch.float32)
         if self.softcap is not None:
             ops.softcap_(logits, self.softcap)
         return logits
+
+
+EMBEDDINGS.register("scaled_embedding", ScaledEmbedding)
+HEADS.register("lm_head", LMHead)

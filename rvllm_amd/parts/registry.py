@@ -1,8 +1,8 @@
 """Registries of part kinds.
 
 Each registry maps a key to a factory ``factory(spec: PartSpec, **context)``.
-A new mixer, feed-forward, norm, position encoding or block arrangement is
-added by registering it; no file of the framework changes.
+A new mixer, feed-forward, norm, position encoding, block arrangement,
+embedding or head is added by registering it; no file of the framework changes.
 """
 
 from __future__ import annotations
@@ -53,3 +53,5 @@ FEED_FORWARDS: Registry = Registry("feed-forward")
 NORMS: Registry = Registry("norm")
 POSITION_ENCODINGS: Registry = Registry("position encoding")
 BLOCKS: Registry = Registry("block arrangement")
+EMBEDDINGS: Registry = Registry("embedding")
+HEADS: Registry = Registry("head")

@@ -68,6 +68,7 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     prefix: str = "model"
+    final_norm_name: str = "norm"  # the final norm's tensor is <prefix>.<final_norm_name>.weight
 
     def __post_init__(self):
         n = len(self.layers)

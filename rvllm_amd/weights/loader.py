@@ -16,17 +16,13 @@ from __future__ import annotations
 
 import os
 import warnings
-from typing import Iterable, Sequence
+from pathlib import Path
+from typing import Sequence
 
 import torch
 
 from ..parts.base import ParamSpec
-from .safetensors_io import SafetensorsError, SafetensorsFile, resolve_shards
-
-# Prefixes under which a checkpoint may keep the text decoder
-# (v3/crates/rvllm-loader/src/gemma4_arch.rs:624-658).
-KNOWN_PREFIXES = ("model.language_model", "language_model.model", "language_model", "model")
-
+from .safetensors_io import SafetensorsError, SafetensorsFile, read_shard_index, resolve_shards
 
 class WeightError(ValueError):
     """Everything that is wrong with a folder's tensors, in one message."""
@@ -51,17 +47,22 @@ class WeightError(ValueError):
         super().__init__("\n".join(lines))
 
 
-def detect_prefix(names: Iterable[str]) -> str:
-    """The prefix under which ``embed_tokens.weight`` is stored."""
-    names = set(names)
-    for prefix in KNOWN_PREFIXES:
-        if f"{prefix}.embed_tokens.weight" in names:
-            return prefix
-    return "model"
-
-
 def open_model_files(model_dir: str | os.PathLike) -> list[SafetensorsFile]:
-    return [SafetensorsFile(p) for p in resolve_shards(model_dir)]
+    """The folder's safetensors files, opened.  Where an index says which file
+    holds which tensor, every tensor must lie in the file the index names."""
+    files = [SafetensorsFile(p) for p in resolve_shards(model_dir)]
+    weight_map = read_shard_index(model_dir)
+    if weight_map is not None:
+        root = Path(model_dir).resolve()
+        held = {f.path.resolve(): set(f.names()) for f in files}
+        astray = [f"{name!r} is not in {fname}" for name, fname in weight_map.items()
+                  if name not in held.get((root / fname).resolve(), ())]
+        if astray:
+            for f in files:
+                f.close()
+            raise SafetensorsError(f"{model_dir}: the shard index names tensors that their files do not hold: "
+                                   + "; ".join(astray[:8]) + (" ..." if len(astray) > 8 else ""))
+    return files
 
 
 def tensor_names(files: Sequence[SafetensorsFile]) -> list[str]:

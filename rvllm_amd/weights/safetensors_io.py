@@ -145,24 +145,40 @@ class SafetensorsFile:
         self._fh.close()
 
 
+def read_shard_index(model_dir: str | os.PathLike) -> Optional[dict[str, str]]:
+    """tensor name -> file name from model.safetensors.index.json, or None when the folder has no index.
+    File names must be plain relative paths that stay inside the folder
+    (v3/crates/rvllm-loader/src/safetensors.rs:325-421)."""
+    root = Path(model_dir).resolve()
+    index = root / "model.safetensors.index.json"
+    if not index.is_file():
+        return None
+    try:
+        doc = json.loads(index.read_text(), object_pairs_hook=_no_duplicates)
+        weight_map = doc["weight_map"]
+        assert isinstance(weight_map, dict)
+    except (json.JSONDecodeError, KeyError, AssertionError, SafetensorsError) as e:
+        raise SafetensorsError(f"{index}: not a valid shard index: {e}") from None
+    for name, fname in weight_map.items():
+        if not isinstance(fname, str) or not fname:
+            raise SafetensorsError(f"{index}: the file of tensor {name!r} is no file name: {fname!r}")
+        parts = Path(fname).parts
+        if Path(fname).is_absolute() or any(part in ("..", ".") for part in parts) or \
+                root not in (root / fname).resolve().parents:
+            raise SafetensorsError(f"{index}: shard {fname!r} leaves the model folder")
+    return weight_map
+
+
 def resolve_shards(model_dir: str | os.PathLike) -> list[Path]:
     """The safetensors files of a model folder."""
     root = Path(model_dir).resolve()
-    index = root / "model.safetensors.index.json"
-    if index.is_file():
-        try:
-            doc = json.loads(index.read_text(), object_pairs_hook=_no_duplicates)
-            weight_map = doc["weight_map"]
-            assert isinstance(weight_map, dict)
-        except (json.JSONDecodeError, KeyError, AssertionError, SafetensorsError) as e:
-            raise SafetensorsError(f"{index}: not a valid shard index: {e}") from None
+    weight_map = read_shard_index(root)
+    if weight_map is not None:
         files = []
         for fname in dict.fromkeys(weight_map.values()):
             p = (root / fname).resolve()
-            if not isinstance(fname, str) or root not in p.parents:
-                raise SafetensorsError(f"{index}: shard {fname!r} leaves the model folder")
             if not p.is_file():
-                raise SafetensorsError(f"{index}: shard {fname!r} not found")
+                raise SafetensorsError(f"{root / 'model.safetensors.index.json'}: shard {fname!r} not found")
             files.append(p)
         return files
     single = root / "model.safetensors"

@@ -142,6 +142,16 @@ def find_prefix(weights: dict) -> str:
     raise KeyError("no embed_tokens.weight found")
 
 
+def find_head(weights: dict) -> str:
+    """An untied head: ``lm_head.weight`` under no prefix, as the reference
+    looks it up (v3/crates/rvllm-loader/src/gemma4_load.rs:431-436), or beside
+    a nested decoder."""
+    for name in ("lm_head.weight", "language_model.lm_head.weight", "model.lm_head.weight"):
+        if name in weights:
+            return name
+    raise KeyError("no lm_head.weight found")
+
+
 def layer(x, positions, w: dict, p: str, cfg: dict, kind: str) -> torch.Tensor:
     """One decoder layer on a whole sequence x[T, H], in the order of
     v3/crates/rvllm-loader/src/metal_host.rs:492-628: input norm, q/k/v,
@@ -190,7 +200,7 @@ def forward(weights: dict, cfg: dict, token_ids, dtype=torch.float32) -> torch.T
     for l in range(cfg["layers"]):
         x = layer(x, positions, w, f"{pre}.layers.{l}", cfg, cfg["kinds"][l])
     x = rmsnorm(x, w[f"{pre}.norm.weight"], cfg["eps"])
-    head = emb if cfg["tied"] else w["lm_head.weight"]
+    head = emb if cfg["tied"] else w[find_head(w)]
     logits = x @ head.T
     if cfg["softcap"] is not None:
         logits = softcap(logits, cfg["softcap"])
@@ -205,14 +215,23 @@ def load_weights(model_dir) -> dict:
     return load_file(str(Path(model_dir) / "model.safetensors"))
 
 
+def pick_greedy(row: torch.Tensor) -> int:
+    """The id of the largest logit of a row; equal maxima give the lowest id:
+    the reference scans from the left with a strict ``>``
+    (kernels/argmax.cu:16-25, v3/crates/rvllm-fused/src/reference.rs:200-225)."""
+    best, best_value = 0, None
+    for i, value in enumerate(row.tolist()):
+        if best_value is None or value > best_value:
+            best, best_value = i, value
+    return best
+
+
 def greedy(weights: dict, cfg: dict, prompt, steps: int, dtype=torch.float32) -> list[int]:
-    """Greedy continuation by re-running the whole sequence every step;
-    equal maxima give the lowest id (kernels/argmax.cu:16-25)."""
+    """Greedy continuation by re-running the whole sequence every step."""
     ids = list(prompt)
     out = []
     for _ in range(steps):
-        row = forward(weights, cfg, ids, dtype)[-1]
-        best = int(torch.nonzero(row == row.max())[0])
+        best = pick_greedy(forward(weights, cfg, ids, dtype)[-1])
         out.append(best)
         ids.append(best)
     return out

@@ -17,8 +17,9 @@ from rvllm_amd.engine.batch import BatchBuilder, Portion
 from rvllm_amd.engine.runner import ModelRunner
 from rvllm_amd.kernels import ops
 from rvllm_amd.models import Architecture, register_architecture, unregister_architecture
-from rvllm_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, FeedForward, LayerSpec, Mixer,
-                             ModelSpec, ParamSpec, PartSpec, PositionEncoding, ScheduleEntry, StateNeed)
+from rvllm_amd.parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS, Embedding,
+                             FeedForward, Head, LayerSpec, Mixer, ModelSpec, ParamSpec, PartSpec, PositionEncoding,
+                             ScheduleEntry, StateNeed)
 from rvllm_amd.parts.linear import linear
 from rvllm_amd.weights.random_init import random_tensors, write_random_model
 
@@ -175,7 +176,10 @@ def test_block_part_is_the_plain_layer(plain_models):
 class RunningMeanMixer(Mixer):
     """y[t] = W @ mean(x[0..t]): keeps the running sum and the count of a
     request in a slot of fixed size, portions must continue where the slot
-    left off."""
+    left off.  It reads the step's slots on the host and launches by what it finds there, so its work
+    cannot be recorded into a graph: it says so, and the runner then never takes a step from one."""
+
+    capturable = False
 
     def __init__(self, spec, *, hidden_size):
         self.hidden = hidden_size
@@ -436,3 +440,125 @@ def test_toy_routed_feed_forward_and_position_encoding_plug_in(tmp_path):
         unregister_architecture("Toy2ForCausalLM")
         FEED_FORWARDS.unregister("top_one_experts")
         POSITION_ENCODINGS.unregister("root_positions")
+
+
+def test_a_part_that_cannot_be_recorded_keeps_its_model_out_of_graphs(tmp_path, toy_architecture):
+    """The toy mixer waits for the device inside its forward.  In bf16 with graphs switched on (the default)
+    decode steps of its model run kernel by kernel; the same engine replays graphs for a model whose parts all
+    can be recorded."""
+    cfg = ToyConfig("ToyForCausalLM", hidden=24, vocab=50, layers=3)
+    folder = write_random_model(tmp_path / "toy", cfg, seed=7, dtype=torch.bfloat16)
+    engine_cfg = EngineConfig(dtype="bfloat16", max_model_len=128, max_num_seqs=3, max_num_batched_tokens=128,
+                              max_prefill_chunk=128, max_cache_tokens=256, use_graphs=True)
+    runner = ModelRunner.from_model_dir(folder, engine_cfg)
+    assert not runner.model.capturable
+    weights = P.load_weights(folder)
+    ids = [3, 14, 15, 9, 26, 5, 35, 8, 9, 7, 9, 3]
+    want = toy_plain(weights, cfg, ids)
+    runner.add_request("a")
+    got = [runner.step([("a", ids[:4], list(range(4)))]).float().cpu()]
+    for t in ids[4:]:  # decoded one by one: steps that a model of recordable parts would take from a graph
+        got.append(runner.step([("a", [t], [0])]).float().cpu())
+    assert runner.graph_replays == 0
+    got = torch.cat(got).double()
+    assert (got - want).abs().max() <= 3e-2 * want.abs().max()
+
+
+# --------------------------------------------------------------------------
+# A toy embedding (token table plus a learned table of absolute positions) and a toy head (with a bias),
+# registered from here: the model builds both through the registries.
+# --------------------------------------------------------------------------
+class TokenAndPositionEmbedding(Embedding):
+    def __init__(self, spec, *, hidden_size, vocab_size):
+        self.hidden, self.vocab, self.positions = hidden_size, vocab_size, int(spec["positions"])
+
+    def param_specs(self, prefix):
+        return [ParamSpec(f"{prefix}.wte.weight", (self.vocab, self.hidden), init=("normal", 0.5)),
+                ParamSpec(f"{prefix}.wpe.weight", (self.positions, self.hidden), init=("normal", 0.5))]
+
+    def bind(self, tensors, prefix, device, dtype):
+        self.table = tensors[f"{prefix}.wte.weight"].to(device=device, dtype=dtype).contiguous()
+        self.places = tensors[f"{prefix}.wpe.weight"].to(device=device, dtype=dtype).contiguous()
+
+    def forward(self, step, out):
+        ops.embed_gather(self.table, step.token_ids, 1.0, out)  # the framework's kernel, twice
+        places = torch.empty_like(out)
+        ops.embed_gather(self.places, step.positions, 1.0, places)
+        return out.add_(places)
+
+
+class BiasedHead(Head):
+    def __init__(self, spec, *, hidden_size, vocab_size, embedding):
+        self.hidden, self.vocab, self.embedding = hidden_size, vocab_size, embedding
+
+    def param_specs(self, prefix):
+        return [ParamSpec("out_bias", (self.vocab,), init=("normal", 1.0))]
+
+    def bind(self, tensors, prefix, device, dtype):
+        self.bias = tensors["out_bias"].to(device=device, dtype=torch.float32)
+
+    def forward(self, x):
+        return linear(x, self.embedding.table, out_dtype=torch.float32).add_(self.bias)
+
+
+def toy3_spec(cfg: ToyConfig, prefix="model") -> ModelSpec:
+    norm = PartSpec("rmsnorm", {"eps": 1e-6, "unit_offset": False})
+    attn = PartSpec("attention", {"num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "scale": 0.25, "window": None,
+                                  "qk_norm": None, "position": None})  # positions come from the embedding alone
+    ff = PartSpec("gated_mlp", {"intermediate_size": 2 * cfg.hidden, "activation": "silu"})
+    layers = tuple(LayerSpec(f"{prefix}.h.{l}", PartSpec("sandwich"), attn, ff, norm) for l in range(cfg.layers))
+    return ModelSpec(cfg.architecture, cfg.hidden, cfg.vocab, 64, PartSpec("token_and_position", {"positions": 64}),
+                     layers, tuple(ScheduleEntry(l) for l in range(cfg.layers)), norm, PartSpec("biased_head"), prefix,
+                     final_norm_name="ln_f")
+
+
+def toy3_plain(weights, cfg: ToyConfig, ids):
+    w = {k: v.double() for k, v in weights.items()}
+    norm = lambda x, name: x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6) * w[name]
+    T = len(ids)
+    x = w["model.wte.weight"][ids] + w["model.wpe.weight"][:T]
+    for l in range(cfg.layers):
+        p = f"model.h.{l}"
+        h = norm(x, f"{p}.input_layernorm.weight")
+        q, k, v = ((h @ w[f"{p}.self_attn.{n}_proj.weight"].T).view(T, -1, 16) for n in "qkv")
+        a = P.attention(q, k, v, 0.25, None).reshape(T, 32) @ w[f"{p}.self_attn.o_proj.weight"].T
+        x = x + norm(a, f"{p}.post_attention_layernorm.weight")
+        h = norm(x, f"{p}.pre_feedforward_layernorm.weight")
+        f = (torch.nn.functional.silu(h @ w[f"{p}.mlp.gate_proj.weight"].T) * (h @ w[f"{p}.mlp.up_proj.weight"].T)) \
+            @ w[f"{p}.mlp.down_proj.weight"].T
+        x = x + norm(f, f"{p}.post_feedforward_layernorm.weight")
+    return norm(x, "model.ln_f.weight") @ w["model.wte.weight"].T + w["out_bias"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_embedding_and_head_plug_in_and_replay_from_graphs(tmp_path, dtype):
+    EMBEDDINGS.register("token_and_position", TokenAndPositionEmbedding, replace=True)
+    HEADS.register("biased_head", BiasedHead, replace=True)
+    register_architecture(Architecture("Toy3ForCausalLM", ToyConfig.from_dict, toy3_spec, ToyConfig.to_dict), replace=True)
+    try:
+        cfg = ToyConfig("Toy3ForCausalLM", hidden=24, vocab=40, layers=2)
+        store = torch.float32 if dtype == "float32" else torch.bfloat16
+        folder = write_random_model(tmp_path / "toy3", cfg, seed=13, dtype=store)
+        weights = P.load_weights(folder)
+        assert {"model.wte.weight", "model.wpe.weight", "out_bias", "model.ln_f.weight"} <= set(weights)
+        assert not any("embed_tokens" in k or k.startswith("model.norm.") for k in weights)  # its own names only
+        runner = ModelRunner.from_model_dir(folder, EngineConfig(dtype=dtype, max_model_len=64, max_num_seqs=2,
+                                                                max_num_batched_tokens=64, max_prefill_chunk=64,
+                                                                max_cache_tokens=128, use_graphs=True))
+        assert runner.model.capturable
+        ids = [5, 1, 33, 7, 7, 20, 39, 0, 12, 3, 18, 25, 6, 31]
+        want = toy3_plain(weights, cfg, ids)
+        tol = 1e-4 if dtype == "float32" else 3e-2 * want.abs().max().item()
+        runner.add_request("whole")
+        got = runner.step([("whole", ids, list(range(len(ids))))]).float().cpu().double()
+        assert (got - want).abs().max() <= tol
+        runner.add_request("cut")
+        parts = [runner.step([("cut", ids[:6], list(range(6)))]).float().cpu()]
+        for t in ids[6:]:
+            parts.append(runner.step([("cut", [t], [0])]).float().cpu())
+        assert (torch.cat(parts).double() - want).abs().max() <= tol
+        assert (runner.graph_replays > 0) == (dtype == "bfloat16")  # positions reach the embedding from the step's arrays
+    finally:
+        unregister_architecture("Toy3ForCausalLM")
+        EMBEDDINGS.unregister("token_and_position")
+        HEADS.unregister("biased_head")

@@ -204,7 +204,132 @@ def test_kinds_follow_the_pattern(plain_models):
 
 
 def test_greedy_takes_the_lowest_id_among_equal_maxima():
-    # kernels/argmax.cu:16-25, pinned by rvllm-invariants/tests/identity.rs:91-128
-    row = torch.tensor([2.0, 9.0, 4.0, 9.0, 1.0])
-    assert int(torch.nonzero(row == row.max())[0]) == 1
-    assert int(torch.nonzero(torch.full((4,), 1.5) == 1.5)[0]) == 0
+    # the reference's golden rows: v3/crates/rvllm-invariants/tests/identity.rs:91-128
+    assert P.pick_greedy(torch.tensor([2.0, 9.0, 4.0, 9.0, 1.0])) == 1
+    assert P.pick_greedy(torch.full((4,), 1.5)) == 0
+    assert P.pick_greedy(torch.tensor([0.1, 0.2, 9.9, 0.3])) == 2
+    assert P.pick_greedy(torch.tensor([7.0, 0.0, 1.0, 2.0])) == 0
+
+
+def test_greedy_generation_feeds_its_choice_back(plain_models):
+    """Each chosen token is the pick of the row the whole sequence so far ends in."""
+    w, cfg = plain_models["A"]
+    prompt = [5, 17, 3]
+    out = P.greedy(w, cfg, prompt, 3)
+    ids = list(prompt)
+    for token in out:
+        assert token == P.pick_greedy(P.forward(w, cfg, ids)[-1])
+        ids.append(token)
+
+
+# ---- what the Gemma-3 decoder has beyond the reference's text, pinned by a second composition -------------
+def library_layer(x, positions, w, p, cfg, kind):
+    """One layer put together from library routines and the other common
+    spelling of the rotation (x cos + rotate_half(x) sin): ``F.rms_norm`` with
+    the gain 1 + w, ``F.scaled_dot_product_attention`` with an explicit band or
+    causal mask, ``F.gelu(approximate="tanh")``.  It shares no line with
+    ``plain_gemma.layer``."""
+    T = x.shape[0]
+    nq, nkv, hd, eps = cfg["nq"], cfg["nkv"], cfg["hd"], cfg["eps"]
+    norm = lambda t, name: F.rms_norm(t, (t.shape[-1],), 1.0 + w[f"{p}.{name}.weight"], eps)
+    h = norm(x, "input_layernorm")
+    q = F.linear(h, w[f"{p}.self_attn.q_proj.weight"]).view(T, nq, hd)
+    k = F.linear(h, w[f"{p}.self_attn.k_proj.weight"]).view(T, nkv, hd)
+    v = F.linear(h, w[f"{p}.self_attn.v_proj.weight"]).view(T, nkv, hd)
+    q, k = norm(q, "self_attn.q_norm"), norm(k, "self_attn.k_norm")
+    theta, factor = (cfg["theta_local"], 1.0) if kind == "sliding" else (cfg["theta_global"], cfg["factor"])
+    # the inverse frequencies are a 32-bit table (rounded once, after the division by the factor)
+    freqs = (1.0 / (theta ** (torch.arange(0, hd, 2, dtype=torch.float64) / hd)) / factor).float().double()
+    angle = torch.outer(positions.double(), freqs)
+    cos, sin = torch.cat([angle.cos()] * 2, -1)[:, None, :], torch.cat([angle.sin()] * 2, -1)[:, None, :]
+    rotate_half = lambda t: torch.cat([-t[..., hd // 2:], t[..., : hd // 2]], -1)
+    q, k = q * cos + rotate_half(q) * sin, k * cos + rotate_half(k) * sin
+    i = torch.arange(T)
+    mask = i[None, :] <= i[:, None]
+    if kind == "sliding":
+        mask &= i[:, None] - i[None, :] < cfg["window"]
+    a = sdpa(q, k, v, cfg["qpas"] ** -0.5, mask).reshape(T, nq * hd)
+    x = x + norm(F.linear(a, w[f"{p}.self_attn.o_proj.weight"]), "post_attention_layernorm")
+    h = norm(x, "pre_feedforward_layernorm")
+    f = F.linear(F.gelu(F.linear(h, w[f"{p}.mlp.gate_proj.weight"]), approximate="tanh")
+                 * F.linear(h, w[f"{p}.mlp.up_proj.weight"]), w[f"{p}.mlp.down_proj.weight"])
+    return x + norm(f, "post_feedforward_layernorm")
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("kind", ["sliding", "global"])
+def test_layer_equals_a_composition_of_library_routines(plain_models, name, kind):
+    w, cfg = plain_models[name]
+    w = {k: v.double() for k, v in w.items()}
+    T = 3 * cfg["window"] + 5 if cfg["window"] < 40 else cfg["window"] + 30  # past every window's edge
+    x = torch.randn(T, cfg["hidden"], dtype=torch.float64)
+    positions = torch.arange(T)
+    got = P.layer(x, positions, w, "model.layers.0", cfg, kind)
+    want = library_layer(x, positions, w, "model.layers.0", cfg, kind)
+    assert torch.allclose(got, want, atol=1e-9)
+
+
+def test_score_scale_is_the_scalar_to_the_power_minus_one_half(plain_models):
+    """Scores are q.k * query_pre_attn_scalar^-1/2 with q normed by the gain
+    1 + w: a scalar four times as large and a query gain twice as large cancel.
+    A scale of 1/scalar, a scale taken from the head size, or a gain of w
+    instead of 1 + w each break the equality."""
+    w, cfg = plain_models["B"]
+    w = {k: v.double() for k, v in w.items()}
+    assert cfg["qpas"] != cfg["hd"]
+    x = torch.randn(12, cfg["hidden"], dtype=torch.float64)
+    pos = torch.arange(12)
+    base = P.layer(x, pos, w, "model.layers.2", cfg, "global")
+    w2 = dict(w)
+    gain = 1.0 + w["model.layers.2.self_attn.q_norm.weight"]
+    w2["model.layers.2.self_attn.q_norm.weight"] = 2.0 * gain - 1.0
+    other = P.layer(x, pos, w2, "model.layers.2", dict(cfg, qpas=4 * cfg["qpas"]), "global")
+    assert torch.allclose(base, other, atol=1e-10)
+    assert not torch.allclose(base, P.layer(x, pos, w, "model.layers.2", dict(cfg, qpas=4 * cfg["qpas"]), "global"),
+                              atol=1e-6)
+
+
+def test_each_layer_kind_reads_its_own_base_and_only_global_layers_scale(plain_models):
+    w, cfg = plain_models["B"]
+    w = {k: v.double() for k, v in w.items()}
+    x = torch.randn(9, cfg["hidden"], dtype=torch.float64)
+    pos = torch.arange(9) + 40
+    run = lambda c, kind: P.layer(x, pos, w, "model.layers.0", c, kind)
+    # a sliding layer knows nothing of the global base or the factor; a global one nothing of the local base
+    assert torch.equal(run(cfg, "sliding"), run(dict(cfg, theta_global=123.0, factor=9.0), "sliding"))
+    assert torch.equal(run(cfg, "global"), run(dict(cfg, theta_local=123.0, window=2), "global"))
+    assert not torch.allclose(run(cfg, "global"), run(dict(cfg, theta_global=123.0), "global"), atol=1e-6)
+    assert not torch.allclose(run(cfg, "sliding"), run(dict(cfg, theta_local=123.0), "sliding"), atol=1e-6)
+    # the factor divides the positions of a global layer: factor 4 at positions 4p is factor 1 at positions p
+    a = P.layer(x, 4 * torch.arange(9), w, "model.layers.0", cfg, "global")
+    b = P.layer(x, torch.arange(9), w, "model.layers.0", dict(cfg, factor=1.0), "global")
+    assert cfg["factor"] == 4.0 and torch.allclose(a, b, atol=1e-10)
+
+
+def test_query_and_key_norm_come_before_the_rotation(plain_models):
+    """With gains that differ inside a rotated pair, norming after the rotation
+    would make scores depend on the positions themselves; normed first, only
+    distances count, under any gains."""
+    w, cfg = plain_models["B"]
+    w = {k: v.double() for k, v in w.items()}
+    g = torch.Generator().manual_seed(4)
+    for n in ("q_norm", "k_norm"):
+        w[f"model.layers.2.self_attn.{n}.weight"] = torch.randn(cfg["hd"], generator=g, dtype=torch.float64)
+    x = torch.randn(7, cfg["hidden"], dtype=torch.float64, generator=g)
+    a = P.layer(x, torch.arange(7), w, "model.layers.2", cfg, "global")
+    b = P.layer(x, torch.arange(7) + 333, w, "model.layers.2", cfg, "global")
+    assert torch.allclose(a, b, atol=1e-9)
+
+
+def test_the_untied_head_is_its_own_matrix(plain_models):
+    w, cfg = plain_models["A"]
+    w = {k: v.float().clone() for k, v in w.items()}
+    ids = [9, 8, 7, 6]
+    tied = P.forward(w, cfg, ids)
+    head = torch.randn(cfg["vocab"], cfg["hidden"], generator=torch.Generator().manual_seed(8)) * 0.02
+    for name in ("lm_head.weight", "language_model.lm_head.weight"):
+        untied = P.forward(dict(w, **{name: head}), dict(cfg, tied=False), ids)
+        # the same final hidden state against another matrix: the input side still reads the embedding table
+        x = torch.linalg.lstsq(w["model.embed_tokens.weight"].double(), tied.double().T).solution.T  # hidden rows
+        assert torch.allclose(untied.double(), x @ head.double().T, atol=1e-4)
+    assert not torch.allclose(untied, tied, atol=1e-3)

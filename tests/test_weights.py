@@ -10,7 +10,8 @@ import torch
 import tiny_models
 from rvllm_amd.models import DecoderModel, load_config
 from rvllm_amd.parts.base import ParamSpec
-from rvllm_amd.weights.loader import WeightError, detect_prefix, load_tensors, open_model_files, tensor_names
+from rvllm_amd.models.gemma3 import locate_tensors
+from rvllm_amd.weights.loader import WeightError, load_tensors, open_model_files, tensor_names
 from rvllm_amd.weights.safetensors_io import SafetensorsError, SafetensorsFile, resolve_shards, write_safetensors
 
 
@@ -97,7 +98,7 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path, model_dir
     save_file(tensors, str(tmp_path / "model.safetensors"))
     arch, cfg = load_config(tmp_path)
     files = open_model_files(tmp_path)
-    model = DecoderModel(arch.build_spec(cfg, detect_prefix(tensor_names(files))))
+    model = DecoderModel(arch.build_spec(cfg, **arch.locate_tensors(tensor_names(files))))
     with pytest.raises(WeightError) as e:
         load_tensors(files, model.param_specs(), torch.bfloat16, source=str(tmp_path))
     err = e.value
@@ -132,9 +133,21 @@ def test_kept_types(tmp_path):
 
 
 def test_prefix_detection():
-    assert detect_prefix(["model.language_model.embed_tokens.weight"]) == "model.language_model"
-    assert detect_prefix(["language_model.model.embed_tokens.weight"]) == "language_model.model"
-    assert detect_prefix(["model.embed_tokens.weight", "x"]) == "model"
+    assert locate_tensors(["model.language_model.embed_tokens.weight"])["prefix"] == "model.language_model"
+    assert locate_tensors(["language_model.model.embed_tokens.weight"])["prefix"] == "language_model.model"
+    assert locate_tensors(["model.embed_tokens.weight", "x"]) == {"prefix": "model", "head_weight": "lm_head.weight"}
+
+
+def test_an_untied_head_is_found_beside_a_nested_decoder():
+    # as the reference looks it up: under no prefix (gemma4_load.rs:431-436)
+    assert locate_tensors(["model.language_model.embed_tokens.weight", "lm_head.weight"])["head_weight"] == "lm_head.weight"
+    # beside the decoder it belongs to
+    assert locate_tensors(["language_model.model.embed_tokens.weight", "language_model.lm_head.weight"])[
+        "head_weight"] == "language_model.lm_head.weight"
+    assert locate_tensors(["language_model.embed_tokens.weight", "language_model.lm_head.weight"])[
+        "head_weight"] == "language_model.lm_head.weight"
+    # none there: the plain name, which the loader then reports missing
+    assert locate_tensors(["model.embed_tokens.weight"])["head_weight"] == "lm_head.weight"
 
 
 def test_nested_prefix_loads_and_ignores_the_vision_part(tmp_path, model_dirs):
@@ -147,9 +160,10 @@ def test_nested_prefix_loads_and_ignores_the_vision_part(tmp_path, model_dirs):
     save_file(tensors, str(tmp_path / "model.safetensors"))
     arch, cfg = load_config(tmp_path)
     files = open_model_files(tmp_path)
-    prefix = detect_prefix(tensor_names(files))
-    model = DecoderModel(arch.build_spec(cfg, prefix))
-    got = load_tensors(files, model.param_specs(), torch.bfloat16, ignore=("model.vision_tower.",))
+    where = arch.locate_tensors(tensor_names(files))
+    prefix = where["prefix"]
+    model = DecoderModel(arch.build_spec(cfg, **where))
+    got = load_tensors(files, model.param_specs(), torch.bfloat16, ignore=arch.ignored_prefixes)
     assert f"{prefix}.layers.1.mlp.down_proj.weight" in got and len(got) == 28
 
 
