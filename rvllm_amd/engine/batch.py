@@ -144,7 +144,9 @@ class BatchBuilder:
         np.cumsum(lens, out=first[1:])
         tok[:T] = np.concatenate([np.asarray(p.tokens, dtype=np.int32) for p in portions]) if T else 0
         req[:T] = np.repeat(np.arange(B, dtype=np.int32), lens)
-        pos[:T] = np.arange(T, dtype=np.int64) + np.repeat(starts - first[:B], lens)
+        place = np.repeat(starts - first[:B], lens)
+        place += np.arange(T, dtype=np.int64)  # in place, as for the tables below
+        pos[:T] = place
         qs[: B + 1] = first
         cs[:B] = starts
         cl[:B] = starts + lens
@@ -173,7 +175,10 @@ class BatchBuilder:
                 # entry j of row b goes to b * width + j
                 row_first = np.zeros(B, dtype=np.int64)
                 np.cumsum(counts[:-1], out=row_first[1:])
-                where = np.arange(total, dtype=np.int64) + np.repeat(np.arange(B, dtype=np.int64) * width - row_first, counts)
+                # added in place: a sum of two temporaries of 256 KB or more makes numpy look up the call stack
+                # to see whether it may reuse one of them, which costs some 100 ms the first time it happens
+                where = np.repeat(np.arange(B, dtype=np.int64) * width - row_first, counts)
+                where += np.arange(total, dtype=np.int64)
                 dst[where] = np.concatenate(held)
         self.dev.copy_(self.host, non_blocking=True)
         if event is not None:

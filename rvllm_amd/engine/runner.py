@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import collections
 import dataclasses
+import gc
 import os
 import warnings
 from typing import Hashable, Optional, Sequence
@@ -64,6 +65,11 @@ class ModelRunner:
         self._graphs: collections.OrderedDict[tuple[int, int], tuple] = collections.OrderedDict()
         self._graph_pool = None
         self.graph_replays = 0
+        # What exists now (the interpreter's modules, the model) lives as long as the engine: taken out of the
+        # garbage collector's sight, so that a full collection between two steps, which would walk all of it
+        # (some 100 ms with the libraries loaded here), has almost nothing to walk.
+        gc.collect()
+        gc.freeze()
 
     # ---- decode steps from captured graphs -------------------------------
     GRAPH_CONTEXT_BUCKET = 1024
