@@ -41,6 +41,9 @@ class EngineConfig:
     # Greedy decode steps that may follow one another without the host in between, while nothing waits to be
     # admitted and no request can end by its length on the way (1 = every step is planned by itself).
     greedy_steps_ahead: int = 4
+    # Keep the bf16 matrices a second time, in tiles, for the products of decode steps (up to 64 rows): they then
+    # read a matrix as contiguous streams and take a tenth to a quarter less time; the weights take twice the memory.
+    tiled_weights: bool = True
 
     @property
     def torch_dtype(self) -> torch.dtype:

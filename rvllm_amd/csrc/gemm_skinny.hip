@@ -4,9 +4,14 @@
 // kernel is laid out around that read:
 //
 //   * a wave owns 16 rows of W; W is the A operand of MFMA 16x16x32 (16 rows x
-//     32 k) and is read straight from memory in operand order, 64 contiguous
-//     bytes of a row per load instruction, several steps ahead of the products
-//     that use them;
+//     32 k) and is read straight from memory in operand order, several steps
+//     ahead of the products that use them.  From a matrix stored row by row a
+//     load instruction takes 64 contiguous bytes of each of 16 rows.  A matrix
+//     stored in tiles (rv_tile_weight: the 16 x 32 values of one product
+//     contiguous in the order the lanes hold them, a wave's tiles one after
+//     the other along K) is read as one contiguous stream per wave, 1 KB an
+//     instruction: the memory then sees long runs instead of 64-byte pieces
+//     5 KB apart, and a product takes a tenth to a quarter less time;
 //   * the waves of a block own neighbouring rows and the same range of K, so
 //     they share x: the block stages x through LDS in pieces of 512 (or 256) columns
 //     (double-buffered, rows padded against bank conflicts) and every wave
@@ -36,12 +41,15 @@ union SkFrag {
 // fragment sets in registers): with a memory latency of a few microseconds and
 // a step worth 4 KB a wave, that is what it takes for some 1024 waves to draw
 // the full bandwidth, and it lets a short slice issue all of its loads at once.
-// x is staged one ring's worth of columns at a time (SK_DEPTH * 128), two
-// buffers; for more than 32 rows of x the ring is shorter so that the buffers
-// stay inside LDS.  Rows of the staged x are padded by 8 elements: the row
-// stride is then 4 banks off a multiple of 64 banks, and the 16 lanes that
-// read the same columns of 16 rows hit 64 different banks.
-#define SK_DEPTH_OF(MT) ((MT) <= 2 ? 4 : 2)
+// x is staged a chunk of SK_CHUNK_STEPS steps at a time, two buffers.  Up to 32
+// rows of x a chunk is the whole ring (512 columns); for more rows it is half
+// the ring (256 columns), so that the buffers stay at 67 KB and two blocks fit
+// a CU, and the loop is written out for two chunks so that every place of the
+// ring is still named at compile time.  Rows of the staged x are padded by 8
+// elements: the row stride is then 4 banks off a multiple of 64 banks, and the
+// 16 lanes that read the same columns of 16 rows hit 64 different banks.
+#define SK_DEPTH 4
+#define SK_CHUNK_STEPS_OF(MT) ((MT) <= 2 ? 4 : 2)
 #define SK_MAX_WAVES 8
 
 template <typename TC>
@@ -63,13 +71,16 @@ __device__ __forceinline__ void sk_store1<uint16_t>(uint16_t* p, float a) {
 // values a row (the sums rounded to bf16 first, exactly as the separate kernel
 // for it would read them): a kernel and a pass over memory less, at no cost.
 // A sliced product stores its partial sums as for ACT < 0.
-template <int MT, typename TC, int ACT = -1>
+// TILED: W is stored in tiles (see rv_tile_weight); ldw is then unused.
+template <int MT, typename TC, int ACT = -1, bool TILED = false>
 __global__ void __launch_bounds__(SK_MAX_WAVES * 64)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, TC* __restrict__ out,
                    float* __restrict__ part, int M, int N, int K, long long ldx, long long ldw, long long ldc,
                    int slice_len) {
-  constexpr int DEPTH = SK_DEPTH_OF(MT);
-  constexpr int SK_KC = DEPTH * 128;
+  constexpr int DEPTH = SK_DEPTH;
+  constexpr int CH = SK_CHUNK_STEPS_OF(MT);  // steps of 128 columns in a chunk of x
+  constexpr int UNROLL = DEPTH / CH;         // chunks a pass of the main loop takes
+  constexpr int SK_KC = CH * 128;
   constexpr int SK_ROW = SK_KC + 8;
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][SK_ROW];
   const int tid = threadIdx.x;
@@ -133,13 +144,23 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   for (int mt = 0; mt < MT; ++mt) acc[mt] = (sk_f32x4){0.f, 0.f, 0.f, 0.f};
   const uint16_t* wrow = w + (size_t)row * ldw + kbeg;
   const int last_off = kend - 8 - kbeg;
+  // tiled: this lane's 16 bytes of the wave's tile at K step 0 (a wave past the last rows reads the last tile),
+  // and the steps of 32 a row of tiles has
+  const int k32 = (K + 31) >> 5;
+  const uint16_t* wtile = w + ((size_t)(wave_has_rows ? n0 >> 4 : (N - 1) >> 4) * k32 << 9) + lane * 8;
+  const int step0 = kbeg >> 5;  // slices begin at multiples of 128
 
   SkFrag ring[DEPTH][4];
   auto load_w = [&](int koff, SkFrag* a) {  // koff: offset inside the slice of the 128 columns to read
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int off = koff + j * 32 + kb * 8;
-      a[j].u4 = *(const uint4*)(wrow + (off < last_off ? off : last_off));
+      if constexpr (TILED) {
+        const int ks = step0 + (koff >> 5) + j;
+        a[j].u4 = *(const uint4*)(wtile + ((size_t)(ks < k32 ? ks : k32 - 1) << 9));
+      } else {
+        const int off = koff + j * 32 + kb * 8;
+        a[j].u4 = *(const uint4*)(wrow + (off < last_off ? off : last_off));
+      }
     }
   };
   // The first chunk of x and the whole ring are requested together.  The order
@@ -157,27 +178,35 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
 
   int c = 0;
   do {  // a slice has at least one chunk; a loop that may run zero times lets the first reads sink below the barrier
-    const int buf = c & 1;
-    stage_load(c + 1);  // in flight while this chunk is multiplied
-    asm volatile("" ::: "memory");  // issued before the ring's reads, so that waiting for it leaves those in flight
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
+    for (int u = 0; u < UNROLL; ++u) {
+      // chunk c + u: its x lies in buffer `buf`, its W in the ring's places u * CH .. u * CH + CH - 1.  A chunk
+      // past the slice's end (an odd number of chunks, two a pass) meets zeros of x.
+      const int cc = c + u;
+      const int buf = UNROLL == 1 ? (c & 1) : (u & 1);
+      stage_load(cc + 1);  // in flight while this chunk is multiplied
+      asm volatile("" ::: "memory");  // issued before the ring's reads, so that waiting for it leaves those in flight
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int col = d * 128 + j * 32 + kb * 8;
+      for (int st = 0; st < CH; ++st) {
+        const int d = u * CH + st;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          SkFrag b;
-          b.u4 = *(const uint4*)(&xs[buf][mt * 16 + r16][col]);
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[d][j].v, b.v, acc[mt], 0, 0, 0);
+        for (int j = 0; j < 4; ++j) {
+          const int col = st * 128 + j * 32 + kb * 8;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            SkFrag b;
+            b.u4 = *(const uint4*)(&xs[buf][mt * 16 + r16][col]);
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[d][j].v, b.v, acc[mt], 0, 0, 0);
+          }
         }
+        load_w((cc + UNROLL) * SK_KC + st * 128, ring[d]);  // the same place of the ring, a ring's length on
+        asm volatile("" ::: "memory");                     // here, and not gathered at the chunk's end
       }
-      load_w((c + 1) * SK_KC + d * 128, ring[d]);  // the same place of the ring, one chunk on
-      asm volatile("" ::: "memory");               // here, and not gathered at the chunk's end
+      stage_store(cc + 1, buf ^ 1);  // that buffer was last read in chunk cc - 1, before the barrier below
+      __syncthreads();
     }
-    stage_store(c + 1, buf ^ 1);  // that buffer was last read in chunk c - 1, before the barrier below
-    __syncthreads();
-  } while (++c < chunks);
+    c += UNROLL;
+  } while (c < chunks);
 
   if (!wave_has_rows) return;
   // a lane holds the sums for x row m = mt*16 + r16 and W rows n0 + kb*4 .. + 3
@@ -291,12 +320,17 @@ extern "C" int rv_gemm_skinny_slices(int N, int K) {
 
 template <int MT, typename TC, int ACT = -1>
 static int sk_launch(hipStream_t stream, const uint16_t* x, const uint16_t* w, TC* out, float* part, int M, int N,
-                     int K, long long ldx, long long ldw, long long ldc, int do_reduce) {
+                     int K, long long ldx, long long ldw, long long ldc, int do_reduce, int tiled) {
   int waves, slices, len;
   rv_gemm_skinny_plan(N, K, &waves, &slices, &len);
   if (slices > 1 && part == nullptr) return rv_fail("gemm_skinny: this shape needs a workspace");
   dim3 grid(rv_div_up(rv_div_up(N, 16), waves), slices);
-  gemm_skinny_kernel<MT, TC, ACT><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc, len);
+  if (tiled)
+    gemm_skinny_kernel<MT, TC, ACT, true><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc,
+                                                                               len);
+  else
+    gemm_skinny_kernel<MT, TC, ACT, false><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw,
+                                                                                ldc, len);
   RV_LAUNCH_CHECK("gemm_skinny");
   if (slices > 1 && do_reduce) {
     const long long total = (long long)M * N;
@@ -309,11 +343,14 @@ static int sk_launch(hipStream_t stream, const uint16_t* x, const uint16_t* w, T
 // With `do_reduce` 0 a sliced product leaves its 32-bit partial sums in `part`
 // ([slices][M][N]) for a consumer that adds them itself, and `out` is not
 // written; an unsliced product always writes `out`.
+// `tiled` != 0: W is what rv_tile_weight made of the [N, K] matrix, and ldw is not used.
 extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, void* out, int out_dtype, float* part,
-                              int M, int N, int K, long long ldx, long long ldw, long long ldc, int do_reduce) {
+                              int M, int N, int K, long long ldx, long long ldw, long long ldc, int do_reduce,
+                              int tiled) {
   RV_CHECK(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
-  RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K and the row strides must be multiples of 8");
-  RV_CHECK(ldx >= K && ldw >= K && ldc >= N, "gemm_skinny: leading dimensions too small");
+  RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && (tiled || ldw % 8 == 0),
+           "gemm_skinny: K and the row strides must be multiples of 8");
+  RV_CHECK(ldx >= K && (tiled || ldw >= K) && ldc >= N, "gemm_skinny: leading dimensions too small");
   RV_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny: operands must be 16-byte aligned");
   if (M == 0) return 0;
   const int mt = rv_div_up(M, 16);
@@ -322,9 +359,9 @@ extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, 
 #define SK_CASE(MTV)                                                                                  \
   case MTV:                                                                                           \
     if (out_dtype == RV_F32)                                                                          \
-      return sk_launch<MTV, float>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc, do_reduce);        \
+      return sk_launch<MTV, float>(stream, xp, wp, (float*)out, part, M, N, K, ldx, ldw, ldc, do_reduce, tiled);        \
     if (out_dtype == RV_BF16)                                                                         \
-      return sk_launch<MTV, uint16_t>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc, do_reduce);  \
+      return sk_launch<MTV, uint16_t>(stream, xp, wp, (uint16_t*)out, part, M, N, K, ldx, ldw, ldc, do_reduce, tiled);  \
     break;
   switch (mt) {
     SK_CASE(1)
@@ -340,11 +377,13 @@ extern "C" int rv_gemm_skinny(hipStream_t stream, const void* x, const void* w, 
 // 2q, 2q + 1, then ups 2q, 2q + 1), `out` is [M, N / 2].  Only for shapes whose plan has one slice
 // (rv_gemm_skinny_slices); act 0: gelu in its tanh form, 1: silu.  Otherwise as rv_gemm_skinny.
 extern "C" int rv_gemm_skinny_gate_up(hipStream_t stream, const void* x, const void* w, void* out, int out_dtype,
-                                      int M, int N, int K, long long ldx, long long ldw, long long ldc, int act) {
+                                      int M, int N, int K, long long ldx, long long ldw, long long ldc, int act,
+                                      int tiled) {
   RV_CHECK(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_gate_up: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   RV_CHECK(N % 4 == 0, "gemm_skinny_gate_up: N=%d must be a multiple of 4 (two gates, two ups)", N);
-  RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny_gate_up: K and the row strides must be multiples of 8");
-  RV_CHECK(ldx >= K && ldw >= K && ldc >= N / 2, "gemm_skinny_gate_up: leading dimensions too small");
+  RV_CHECK(K % 8 == 0 && ldx % 8 == 0 && (tiled || ldw % 8 == 0),
+           "gemm_skinny_gate_up: K and the row strides must be multiples of 8");
+  RV_CHECK(ldx >= K && (tiled || ldw >= K) && ldc >= N / 2, "gemm_skinny_gate_up: leading dimensions too small");
   RV_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny_gate_up: operands must be 16-byte aligned");
   RV_CHECK(act == 0 || act == 1, "gemm_skinny_gate_up: unknown activation %d", act);
   RV_CHECK(rv_gemm_skinny_slices(N, K) == 1, "gemm_skinny_gate_up: the plan for N=%d K=%d has slices", N, K);
@@ -355,12 +394,12 @@ extern "C" int rv_gemm_skinny_gate_up(hipStream_t stream, const void* x, const v
 #define SK_CASE(MTV)                                                                                                \
   case MTV:                                                                                                         \
     if (out_dtype == RV_F32)                                                                                        \
-      return act == 0 ? sk_launch<MTV, float, 0>(stream, xp, wp, (float*)out, nullptr, M, N, K, ldx, ldw, ldc, 1)   \
-                      : sk_launch<MTV, float, 1>(stream, xp, wp, (float*)out, nullptr, M, N, K, ldx, ldw, ldc, 1);  \
+      return act == 0 ? sk_launch<MTV, float, 0>(stream, xp, wp, (float*)out, nullptr, M, N, K, ldx, ldw, ldc, 1, tiled)   \
+                      : sk_launch<MTV, float, 1>(stream, xp, wp, (float*)out, nullptr, M, N, K, ldx, ldw, ldc, 1, tiled);  \
     if (out_dtype == RV_BF16)                                                                                       \
       return act == 0                                                                                               \
-                 ? sk_launch<MTV, uint16_t, 0>(stream, xp, wp, (uint16_t*)out, nullptr, M, N, K, ldx, ldw, ldc, 1)  \
-                 : sk_launch<MTV, uint16_t, 1>(stream, xp, wp, (uint16_t*)out, nullptr, M, N, K, ldx, ldw, ldc, 1); \
+                 ? sk_launch<MTV, uint16_t, 0>(stream, xp, wp, (uint16_t*)out, nullptr, M, N, K, ldx, ldw, ldc, 1, tiled)  \
+                 : sk_launch<MTV, uint16_t, 1>(stream, xp, wp, (uint16_t*)out, nullptr, M, N, K, ldx, ldw, ldc, 1, tiled); \
     break;
   switch (mt) {
     SK_CASE(1)
@@ -370,6 +409,41 @@ extern "C" int rv_gemm_skinny_gate_up(hipStream_t stream, const void* x, const v
   }
 #undef SK_CASE
   return rv_fail("gemm_skinny_gate_up: unsupported output dtype %d", out_dtype);
+}
+
+// W [N, K] (row stride ldw) into tiles: tile (n / 16, k / 32) holds 16 rows x 32 columns as the 64 lanes of a
+// product's A operand hold them, lane (k % 32 / 8) * 16 + n % 16 eight consecutive columns, 1 KB a tile, a row of
+// tiles (all of K) contiguous.  Rows past N and columns past K are zeros.  `out` has
+// ceil(N / 16) * ceil(K / 32) * 512 elements.
+__global__ void sk_tile_weight_kernel(const uint16_t* __restrict__ w, uint16_t* __restrict__ out, int N, int K,
+                                      long long ldw, int k32, long long pieces) {
+  const long long p = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // one 16-byte piece of the output
+  if (p >= pieces) return;
+  const int lane = (int)(p & 63);
+  const long long tile = p >> 6;
+  const int ks = (int)(tile % k32);
+  const long long nt = tile / k32;
+  const long long n = nt * 16 + (lane & 15);
+  const int k0 = ks * 32 + (lane >> 4) * 8;
+  uint16_t v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (n < N && k0 + i < K) ? w[n * ldw + k0 + i] : (uint16_t)0;
+  *(uint4*)(out + p * 8) = *(const uint4*)v;
+}
+
+extern "C" long long rv_tile_weight_elements(int N, int K) {
+  return (long long)rv_div_up(N, 16) * rv_div_up(K, 32) * 512;
+}
+
+extern "C" int rv_tile_weight(hipStream_t stream, const void* w, void* out, int N, int K, long long ldw) {
+  RV_CHECK(N > 0 && K > 0 && ldw >= K && w && out, "tile_weight: bad arguments N=%d K=%d", N, K);
+  RV_CHECK(((uintptr_t)out % 16) == 0, "tile_weight: the output must be 16-byte aligned");
+  const int k32 = rv_div_up(K, 32);
+  const long long pieces = rv_tile_weight_elements(N, K) / 8;
+  sk_tile_weight_kernel<<<dim3(rv_div_up(pieces, 256)), dim3(256), 0, stream>>>((const uint16_t*)w, (uint16_t*)out, N, K,
+                                                                              ldw, k32, pieces);
+  RV_LAUNCH_CHECK("tile_weight");
+  return 0;
 }
 
 // out[m][n] (bf16 or 32-bit) = sum over slices of part[s][m][n].

@@ -138,6 +138,37 @@ class SlicedSums:
         return out
 
 
+class TiledWeight:
+    """A bf16 matrix ``[N, K]`` stored for the few-row product: in tiles of 16 rows x 32 columns, each tile's
+    1 KB in the order in which the 64 lanes of a matrix-core product hold it, a row of tiles (all of K)
+    contiguous, so that a wave reads its share of the matrix as one contiguous stream.  ``rows`` is the same
+    matrix row by row, kept for the products that go to the library (more than 64 rows), or None."""
+
+    def __init__(self, rows: torch.Tensor, keep_rows: bool = True):
+        _gpu(rows)
+        _need(rows.dim() == 2 and rows.dtype == torch.bfloat16, "TiledWeight: a bf16 matrix expected")
+        self.n, self.k = rows.shape
+        lib = library()
+        lib.rv_tile_weight_elements.restype = ctypes.c_longlong
+        self.tiles = torch.empty(lib.rv_tile_weight_elements(_c_int(self.n), _c_int(self.k)), dtype=torch.bfloat16,
+                                 device=rows.device)
+        _check(lib.rv_tile_weight(_stream(), _ptr(rows), _ptr(self.tiles), _c_int(self.n), _c_int(self.k),
+                                  _c_ll(rows.stride(0))))
+        self.rows = rows if keep_rows else None
+
+    @property
+    def shape(self):
+        return (self.n, self.k)
+
+    @property
+    def dtype(self):
+        return torch.bfloat16
+
+    @property
+    def device(self):
+        return self.tiles.device
+
+
 def as_tensor(x) -> torch.Tensor:
     """A plain tensor from a tensor or from unreduced ``SlicedSums``."""
     return x.as_tensor() if isinstance(x, SlicedSums) else x
@@ -606,10 +637,11 @@ def topk_select(logits: torch.Tensor, k: int, inv_temp: torch.Tensor) -> tuple[t
     return vals, idx
 
 
-def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+def gemm_bf16(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,
               out_dtype: Optional[torch.dtype] = None, sliced_ok: bool = False):
     """out = x @ w^T on the matrix cores for bf16 inputs; None when no
     hand-written kernel covers the shape (the caller then uses another path).
+    ``w`` is a matrix ``[N, K]`` or a ``TiledWeight``.
 
     Products with up to 64 rows run the kernel that is built around reading
     ``w`` once.  A 32-bit result of more rows (logits at many positions) runs
@@ -617,24 +649,28 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
     library product.  With ``sliced_ok`` a product whose K range is split over
     blocks returns its partial sums as ``SlicedSums`` instead of adding them."""
     m, k = x.shape
+    tiled = isinstance(w, TiledWeight)
     n = w.shape[0]
     out_dtype = out.dtype if out is not None else (out_dtype or x.dtype)
-    if k % 8 or x.stride(1) != 1 or w.stride(1) != 1 or (out is not None and out.stride(1) != 1):
+    if k % 8 or x.stride(1) != 1 or (out is not None and out.stride(1) != 1):
         return None
-    if (m > 1 and x.stride(0) % 8) or (n > 1 and w.stride(0) % 8) or x.data_ptr() % 16 or w.data_ptr() % 16:
+    if (m > 1 and x.stride(0) % 8) or x.data_ptr() % 16:
+        return None
+    if not tiled and (w.stride(1) != 1 or (n > 1 and w.stride(0) % 8) or w.data_ptr() % 16):
         return None
     if m > SKINNY_MAX_ROWS and out_dtype != torch.float32:
         return None
-    _need(x.is_cuda and w.is_cuda, "gemm: arguments must live on the GPU")
+    _need(x.is_cuda and w.device.type == "cuda", "gemm: arguments must live on the GPU")
     _need(w.shape[1] == k and (out is None or out.shape == (m, n)), "gemm: shapes do not fit")
     lib = library()
     ldx = x.stride(0) if m > 1 else k
-    ldw = w.stride(0) if n > 1 else k
+    ldw = 0 if tiled else (w.stride(0) if n > 1 else k)
+    wptr = _ptr(w.tiles if tiled else w)
     slices = lib.rv_gemm_skinny_slices(_c_int(n), _c_int(k))
     if sliced_ok and out is None and slices > 1 and m <= SKINNY_MAX_ROWS:
         part = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
-        _check(lib.rv_gemm_skinny(_stream(), _ptr(x), _ptr(w), None, _dt(x), _ptr(part), _c_int(m), _c_int(n),
-                                  _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(n), _c_int(0)))
+        _check(lib.rv_gemm_skinny(_stream(), _ptr(x), wptr, None, _dt(x), _ptr(part), _c_int(m), _c_int(n),
+                                  _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(n), _c_int(0), _c_int(int(tiled))))
         return SlicedSums(part, out_dtype)
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
@@ -643,10 +679,10 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = No
     part = torch.empty(slices * rows_max * n, dtype=torch.float32, device=x.device) if slices > 1 else None
     for m0 in range(0, m, SKINNY_MAX_ROWS):
         rows = min(SKINNY_MAX_ROWS, m - m0)
-        _check(lib.rv_gemm_skinny(_stream(), ctypes.c_void_p(x.data_ptr() + m0 * ldx * 2), _ptr(w),
+        _check(lib.rv_gemm_skinny(_stream(), ctypes.c_void_p(x.data_ptr() + m0 * ldx * 2), wptr,
                                   ctypes.c_void_p(out.data_ptr() + m0 * ldc * out.element_size()), _dt(out),
                                   _ptr(part), _c_int(rows), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw),
-                                  _c_ll(ldc), _c_int(1)))
+                                  _c_ll(ldc), _c_int(1), _c_int(int(tiled))))
     return out
 
 
@@ -664,27 +700,31 @@ def probe_read(data: torch.Tensor, blocks: int = 2048) -> torch.Tensor:
     return out
 
 
-def gemm_bf16_gate_up(x: torch.Tensor, w_fours: torch.Tensor, activation: str):
+def gemm_bf16_gate_up(x: torch.Tensor, w_fours, activation: str):
     """act(x @ gate^T) * (x @ up^T) in one kernel, for a bf16 ``x`` of at most 64 rows and ``w_fours`` =
-    ``rows_in_fours(gate, up)``: the product applies the activation where it holds the sums, which saves a kernel
-    and a pass over memory.  None when the kernel does not cover the case (rows, alignment, a shape whose product
-    is split along K): the caller then multiplies and applies ``gated_act(..., fours=True)``."""
+    ``rows_in_fours(gate, up)`` (as a matrix or a ``TiledWeight``): the product applies the activation where it
+    holds the sums, which saves a kernel and a pass over memory.  None when the kernel does not cover the case
+    (rows, alignment, a shape whose product is split along K): the caller then multiplies and applies
+    ``gated_act(..., fours=True)``."""
     if x.dtype != torch.bfloat16 or w_fours.dtype != torch.bfloat16:
         return None
     m, k = x.shape
+    tiled = isinstance(w_fours, TiledWeight)
     n = w_fours.shape[0]
-    if m < 1 or m > SKINNY_MAX_ROWS or w_fours.shape[1] != k or k % 8 or n % 4 or x.stride(1) != 1 or w_fours.stride(1) != 1:
+    if m < 1 or m > SKINNY_MAX_ROWS or w_fours.shape[1] != k or k % 8 or n % 4 or x.stride(1) != 1:
         return None
-    if (m > 1 and x.stride(0) % 8) or (n > 1 and w_fours.stride(0) % 8) or x.data_ptr() % 16 or w_fours.data_ptr() % 16:
+    if (m > 1 and x.stride(0) % 8) or x.data_ptr() % 16:
         return None
-    _need(x.is_cuda and w_fours.is_cuda, "gemm: arguments must live on the GPU")
+    if not tiled and (w_fours.stride(1) != 1 or (n > 1 and w_fours.stride(0) % 8) or w_fours.data_ptr() % 16):
+        return None
+    _need(x.is_cuda and w_fours.device.type == "cuda", "gemm: arguments must live on the GPU")
     _need(activation in ACTIVATIONS, f"gemm_bf16_gate_up: unknown activation {activation!r}")
     lib = library()
     if lib.rv_gemm_skinny_slices(_c_int(n), _c_int(k)) != 1:
         return None
     out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
-    _check(lib.rv_gemm_skinny_gate_up(_stream(), _ptr(x), _ptr(w_fours), _ptr(out), _dt(out), _c_int(m), _c_int(n),
-                                      _c_int(k), _c_ll(x.stride(0) if m > 1 else k),
-                                      _c_ll(w_fours.stride(0) if n > 1 else k), _c_ll(n // 2),
-                                      _c_int(ACTIVATIONS[activation])))
+    _check(lib.rv_gemm_skinny_gate_up(_stream(), _ptr(x), _ptr(w_fours.tiles if tiled else w_fours), _ptr(out), _dt(out),
+                                      _c_int(m), _c_int(n), _c_int(k), _c_ll(x.stride(0) if m > 1 else k),
+                                      _c_ll(0 if tiled else (w_fours.stride(0) if n > 1 else k)), _c_ll(n // 2),
+                                      _c_int(ACTIVATIONS[activation]), _c_int(int(tiled))))
     return out

@@ -17,7 +17,7 @@ import torch
 
 from ..kernels import ops
 from .base import KVCacheView, KVNeed, Mixer, ParamSpec
-from .linear import linear
+from .linear import decode_weight, linear
 from .registry import MIXERS, POSITION_ENCODINGS
 from .spec import PartSpec
 
@@ -61,8 +61,8 @@ class PagedAttention(Mixer):
         # q, k and v rows are joined into one matrix, as the reference's loader
         # joins them (v3/crates/rvllm-loader/src/gemma4_load.rs:522,621-625).
         parts = [tensors[f"{p}.{n}_proj.weight"] for n in ("q", "k", "v")]
-        self.w_qkv = torch.cat([t.to(device=device, dtype=dtype) for t in parts], dim=0).contiguous()
-        self.w_o = tensors[f"{p}.o_proj.weight"].to(device=device, dtype=dtype).contiguous()
+        self.w_qkv = decode_weight(torch.cat([t.to(device=device, dtype=dtype) for t in parts], dim=0).contiguous())
+        self.w_o = decode_weight(tensors[f"{p}.o_proj.weight"].to(device=device, dtype=dtype).contiguous())
         if self.qk_norm is not None:
             self.q_norm_w = tensors[f"{p}.q_norm.weight"].to(device).contiguous()
             self.k_norm_w = tensors[f"{p}.k_norm.weight"].to(device).contiguous()

@@ -19,7 +19,7 @@ import torch
 
 from ..kernels import ops
 from .base import Embedding, Head, ParamSpec
-from .linear import linear
+from .linear import decode_weight, linear
 from .registry import EMBEDDINGS, HEADS
 from .spec import PartSpec
 
@@ -70,9 +70,9 @@ class LMHead(Head):
 
     def bind(self, tensors, prefix, device, dtype) -> None:
         if self.tied:
-            self.weight = self.embedding.table
+            self.weight = decode_weight(self.embedding.table)  # the table itself stays row by row for the lookup
         else:
-            self.weight = tensors[self.weight_name].to(device=device, dtype=dtype).contiguous()
+            self.weight = decode_weight(tensors[self.weight_name].to(device=device, dtype=dtype).contiguous())
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = linear(x, self.weight, out_dtype=torch.float32)

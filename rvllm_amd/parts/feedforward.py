@@ -13,7 +13,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, ParamSpec
-from .linear import linear
+from .linear import decode_weight, linear
 from .registry import FEED_FORWARDS
 from .spec import PartSpec
 
@@ -42,8 +42,9 @@ class GatedMLP(FeedForward):
         up = tensors[f"{p}.up_proj.weight"].to(device=device, dtype=dtype)
         # widths that the activation kernel cannot take in fours keep the gates before the ups
         self.fours = self.intermediate_size % ops.FOURS_WIDTH_MULTIPLE == 0
-        self.w_gate_up = ops.rows_in_fours(gate, up) if self.fours else torch.cat([gate, up], dim=0).contiguous()
-        self.w_down = tensors[f"{p}.down_proj.weight"].to(device=device, dtype=dtype).contiguous()
+        self.w_gate_up = decode_weight(ops.rows_in_fours(gate, up) if self.fours
+                                       else torch.cat([gate, up], dim=0).contiguous())
+        self.w_down = decode_weight(tensors[f"{p}.down_proj.weight"].to(device=device, dtype=dtype).contiguous())
 
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
         # a few rows in bf16: the product applies the activation itself where it holds the sums

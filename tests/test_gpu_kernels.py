@@ -152,6 +152,44 @@ def test_gemm_skinny(m, n, k, out_dtype):
     assert torch.equal(one[0], out[m - 1])
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 4096, 2560), (17, 509, 96), (64, 2560, 10240), (33, 100, 2048),
+                                   (3, 20480, 2560), (16, 7, 8), (5, 1000, 1416), (200, 301, 80), (40, 35, 40)])
+def test_a_matrix_stored_in_tiles_gives_the_bits_of_the_matrix_stored_in_rows(m, n, k):
+    """The few-row product reads a matrix either row by row or from tiles of 16 rows x 32 columns laid out in the
+    order its lanes hold them; rows and columns that do not fill a tile (n no multiple of 16, k no multiple of
+    32) are zeros there.  Every sum is the same chain of the same numbers, so the results are equal bit for bit:
+    whole, as unreduced slices, and with the activation in the product."""
+    g = torch.Generator().manual_seed(40)
+    x = dev(torch.randn(m, k, generator=g).bfloat16())
+    w = dev((torch.randn(n, k, generator=g) * 0.05).bfloat16())
+    tiled = ops.TiledWeight(w)
+    assert tiled.shape == (n, k) and tiled.tiles.numel() == -(-n // 16) * -(-k // 32) * 512
+    # the layout itself: tile (i, j), lane (c // 8) * 16 + r, holds w[16 i + r, 32 j + c .. c + 8]
+    t = tiled.tiles.view(-(-n // 16), -(-k // 32), 4, 16, 8).cpu()
+    padded = torch.zeros(-(-n // 16) * 16, -(-k // 32) * 32, dtype=torch.bfloat16)
+    padded[:n, :k] = w.cpu()
+    assert torch.equal(t, padded.view(-(-n // 16), 16, -(-k // 32), 4, 8).permute(0, 2, 3, 1, 4))
+    for out_dtype in (torch.float32, torch.bfloat16):
+        rows = ops.gemm_bf16(x, w, out_dtype=out_dtype)
+        tiles = ops.gemm_bf16(x, tiled, out_dtype=out_dtype)
+        if m > 64 and out_dtype == torch.bfloat16:
+            assert rows is None and tiles is None  # left to the library product, which reads the rows
+            continue
+        assert torch.equal(rows, tiles)
+    if m <= 64:
+        a, b = ops.gemm_bf16(x, w, sliced_ok=True), ops.gemm_bf16(x, tiled, sliced_ok=True)
+        assert type(a) is type(b) and torch.equal(ops.as_tensor(a), ops.as_tensor(b))
+        if n % 4 == 0 and ops.gemm_bf16_gate_up(x, w, "silu") is not None:
+            assert torch.equal(ops.gemm_bf16_gate_up(x, w, "silu"), ops.gemm_bf16_gate_up(x, tiled, "silu"))
+    from rvllm_amd.parts.linear import linear
+    want = x.cpu().double() @ w.cpu().double().T
+    got = linear(x, tiled)  # more than 64 rows: the library's product on the rows kept beside the tiles
+    assert (got.cpu().double() - want).abs().max() <= 1e-2 * max(1.0, want.abs().max().item())
+    if m > 64:
+        with pytest.raises(ops.KernelError, match="row by row"):
+            linear(x, ops.TiledWeight(w, keep_rows=False))
+
+
 @pytest.mark.parametrize("activation", ["gelu_pytorch_tanh", "silu"])
 @pytest.mark.parametrize("m,inter,k", [(1, 40, 64), (8, 96, 128), (64, 10240, 2560), (5, 520, 96), (17, 8, 8)])
 def test_gate_and_up_product_with_the_activation_in_it(m, inter, k, activation):
