@@ -87,16 +87,18 @@ def kv_bytes_per_request(cfg, context: int, elem_bytes: int) -> int:
 
 def attention_flops(cfg, start: int, count: int) -> int:
     """Flops of QK^T and PV for tokens start .. start+count-1 of one request."""
-    total = 0
-    for l in range(cfg.num_hidden_layers):
-        w = cfg.sliding_window if cfg.is_sliding(l) else None
-        # sum over positions p of the number of visible keys
-        if w is None:
-            keys = sum(range(start + 1, start + count + 1))
-        else:
-            keys = sum(min(p + 1, w) for p in range(start, start + count))
-        total += 4 * cfg.num_attention_heads * cfg.head_dim * keys
-    return total
+    def visible(window):  # the number of visible keys, summed over the positions start .. start+count-1
+        total = count * start + count * (count + 1) // 2  # position p sees p + 1 keys
+        if window is not None:
+            # positions from window - 1 on see `window` keys: take off what the others would see beyond it
+            first = max(start, window - 1)
+            n = start + count - first
+            if n > 0:
+                total -= n * first + n * (n + 1) // 2 - n * window
+        return total
+    sliding = sum(1 for l in range(cfg.num_hidden_layers) if cfg.is_sliding(l))
+    keys = sliding * visible(cfg.sliding_window) + (cfg.num_hidden_layers - sliding) * visible(None)
+    return 4 * cfg.num_attention_heads * cfg.head_dim * keys
 
 
 def fill_cache(runner, batch: int, context: int, torch):
@@ -255,24 +257,29 @@ def run_workload(name: str, requests, layers) -> int:
     # (all weights once, the keys and values its tokens may see) and its flops (products, attention, head).
     weight_bytes, layer_flops_per_token, head_flops_per_row = model_numbers(cfg, 2)
     kv_token_bytes = 2 * cfg.kv_size * 2
-    tally = {"steps": 0, "bytes": 0, "flops": 0, "ideal_s": 0.0}
+    planned = []  # every committed step's portions as (start, count, wants a token): priced after the run
     commit = engine.scheduler.commit
 
     def counting_commit(plan, next_tokens):
-        step_bytes, step_flops = weight_bytes, 0
-        for p in plan.portions:
-            for l in range(cfg.num_hidden_layers):
-                seen = p.start + p.count
-                if cfg.is_sliding(l):
-                    seen = min(seen, cfg.sliding_window - 1 + p.count)
-                step_bytes += seen * kv_token_bytes
-            step_flops += p.count * layer_flops_per_token + attention_flops(cfg, p.start, p.count)
-            step_flops += head_flops_per_row if p.wants_token else 0
-        tally["steps"] += 1
-        tally["bytes"] += step_bytes
-        tally["flops"] += step_flops
-        tally["ideal_s"] += max(step_bytes / (PEAK_HBM_GBS * 1e9), step_flops / PEAK_FLOPS["bf16"])
+        planned.append([(p.start, p.count, p.wants_token) for p in plan.portions])
         return commit(plan, next_tokens)
+
+    def price(planned):
+        sliding = sum(1 for l in range(cfg.num_hidden_layers) if cfg.is_sliding(l))
+        full = cfg.num_hidden_layers - sliding
+        tally = {"steps": 0, "bytes": 0, "flops": 0, "ideal_s": 0.0}
+        for portions in planned:
+            step_bytes, step_flops = weight_bytes, 0
+            for start, count, wants in portions:
+                seen = start + count
+                step_bytes += (full * seen + sliding * min(seen, cfg.sliding_window - 1 + count)) * kv_token_bytes
+                step_flops += count * layer_flops_per_token + attention_flops(cfg, start, count)
+                step_flops += head_flops_per_row if wants else 0
+            tally["steps"] += 1
+            tally["bytes"] += step_bytes
+            tally["flops"] += step_flops
+            tally["ideal_s"] += max(step_bytes / (PEAK_HBM_GBS * 1e9), step_flops / PEAK_FLOPS["bf16"])
+        return tally
 
     engine.scheduler.commit = counting_commit
     torch.cuda.synchronize()
@@ -281,6 +288,7 @@ def run_workload(name: str, requests, layers) -> int:
     torch.cuda.synchronize()
     sec = time.perf_counter() - t0
     made = sum(len(r.tokens) for r in results)
+    tally = price(planned)
     print(json.dumps({
         "metric": f"tokens/s through the engine, {name}-sized workload", "value": round((sum(lengths) + made) / sec, 1),
         "unit": "tok/s", "n_gpus": 1, "seconds": round(sec, 2), "higher_is_better": True, "dtype": "bf16",
