@@ -114,13 +114,7 @@ __device__ __forceinline__ void row_store(T* p, const float* in) {
 // V weights starting at element i; the weight vector may be float or bf16.
 template <int V>
 __device__ __forceinline__ void row_load_w(const void* w, int w_f32, int i, float* out) {
-  if (w_f32) {
-#pragma unroll
-    for (int v = 0; v < V; ++v) out[v] = ((const float*)w)[i + v];
-  } else {
-#pragma unroll
-    for (int v = 0; v < V; ++v) out[v] = rv_to_float(((const bf16_t*)w)[i + v]);
-  }
+  rv_load_w_vec<V>(w, w_f32, i, out);
 }
 
 // V values of a branch starting at element i of row `row`: either stored as T,
@@ -344,34 +338,51 @@ extern "C" int rv_add_rmsnorm(hipStream_t stream, const void* branch, int slices
 // gates, then their two ups: gate i at 4 (i / 2) + i % 2, up i two further).
 // ---------------------------------------------------------------------------
 
+// A thread takes GA_ITEMS groups of V outputs, a block's width apart, and asks for all their inputs before it
+// uses the first: at thousands of rows the kernel is a stream of 126 MB, and two 16-byte reads in flight per
+// thread do not draw the memory's full rate.
+#define GA_ITEMS 4
 template <typename T, int V, int ACT, bool FOURS>
 __global__ void gated_act_kernel(const void* __restrict__ gu, int slices, long long slice_stride, T* __restrict__ out,
                                  int inter, long long groups_total) {
-  const long long gidx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (gidx >= groups_total) return;
+  const long long g0 = (long long)blockIdx.x * (blockDim.x * GA_ITEMS) + threadIdx.x;
   const int groups_per_row = inter / V;
-  const long long t = gidx / groups_per_row;
-  const int i = (int)(gidx - t * groups_per_row) * V;
-  float g[V], u[V];
-  if constexpr (FOURS) {  // V is a multiple of 4 here: the thread's outputs are its 2 V neighbouring values
-    const size_t at = (size_t)t * 2 * inter + 2 * (size_t)i;
-    float a[V], b[V];
-    row_load_branch<T, V>(gu, slices, slice_stride, at, a);
-    row_load_branch<T, V>(gu, slices, slice_stride, at + V, b);
+  float a[GA_ITEMS][V], b[GA_ITEMS][V];
+  long long t[GA_ITEMS];
+  int i[GA_ITEMS];
 #pragma unroll
-    for (int v = 0; v < V; ++v) {
-      const int at4 = 4 * (v / 2) + v % 2;  // among the 2 V values
-      g[v] = at4 < V ? a[at4] : b[at4 - V];
-      u[v] = at4 + 2 < V ? a[at4 + 2] : b[at4 + 2 - V];
+  for (int n = 0; n < GA_ITEMS; ++n) {
+    long long gidx = g0 + (long long)n * blockDim.x;
+    gidx = gidx < groups_total ? gidx : groups_total - 1;  // a thread past the end repeats the last group's reads
+    t[n] = gidx / groups_per_row;
+    i[n] = (int)(gidx - t[n] * groups_per_row) * V;
+    if constexpr (FOURS) {  // V is a multiple of 4 here: the thread's outputs are its 2 V neighbouring values
+      const size_t at = (size_t)t[n] * 2 * inter + 2 * (size_t)i[n];
+      row_load_branch<T, V>(gu, slices, slice_stride, at, a[n]);
+      row_load_branch<T, V>(gu, slices, slice_stride, at + V, b[n]);
+    } else {
+      const size_t at = (size_t)t[n] * 2 * inter + i[n];
+      row_load_branch<T, V>(gu, slices, slice_stride, at, a[n]);
+      row_load_branch<T, V>(gu, slices, slice_stride, at + inter, b[n]);
     }
-  } else {
-    const size_t at = (size_t)t * 2 * inter + i;
-    row_load_branch<T, V>(gu, slices, slice_stride, at, g);
-    row_load_branch<T, V>(gu, slices, slice_stride, at + inter, u);
   }
 #pragma unroll
-  for (int v = 0; v < V; ++v) g[v] = rv_gated<T, ACT>(g[v], u[v]);
-  row_store<T, V>(out + (size_t)t * inter + i, g);
+  for (int n = 0; n < GA_ITEMS; ++n) {
+    if (g0 + (long long)n * blockDim.x >= groups_total) break;
+    float g[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      if constexpr (FOURS) {
+        const int at4 = 4 * (v / 2) + v % 2;  // among the 2 V values
+        const float gate = at4 < V ? a[n][at4] : b[n][at4 - V];
+        const float up = at4 + 2 < V ? a[n][at4 + 2] : b[n][at4 + 2 - V];
+        g[v] = rv_gated<T, ACT>(gate, up);
+      } else {
+        g[v] = rv_gated<T, ACT>(a[n][v], b[n][v]);
+      }
+    }
+    row_store<T, V>(out + (size_t)t[n] * inter + i[n], g);
+  }
 }
 
 // `slices` 0: gu holds T values [rows, 2*inter]; otherwise 32-bit partial sums
@@ -386,7 +397,7 @@ extern "C" int rv_gated_act(hipStream_t stream, const void* gu, int slices, long
 #define RV_GA(T, V, A, F)                                                                                          \
   do {                                                                                                             \
     const long long groups = (long long)rows * (inter / V);                                                        \
-    gated_act_kernel<T, V, A, F><<<dim3(rv_div_up(groups, 256)), dim3(256), 0, stream>>>(gu, slices, slice_stride, \
+    gated_act_kernel<T, V, A, F><<<dim3(rv_div_up(groups, 256 * GA_ITEMS)), dim3(256), 0, stream>>>(gu, slices, slice_stride, \
                                                                                         (T*)out, inter, groups);   \
   } while (0)
 #define RV_GA_A(T, V, F)                              \

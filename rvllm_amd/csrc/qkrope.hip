@@ -379,11 +379,8 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
   }
   float g_q[4] = {0.f, 0.f, 0.f, 0.f}, g_k[4] = {0.f, 0.f, 0.f, 0.f};
   if (q_w != nullptr) {  // the same for the whole launch; the weights of queries and keys come together
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      g_q[i] = rv_load_w(q_w, w_f32, d0 + i);
-      g_k[i] = rv_load_w(k_w, w_f32, d0 + i);
-    }
+    rv_load_w_vec<4>(q_w, w_f32, d0, g_q);
+    rv_load_w_vec<4>(k_w, w_f32, d0, g_k);
   }
   const int logical = write_kv != 0 ? pos / page_size : 0;  // without a cache there is no page size either
   const bool in_table = write_kv != 0 && logical < table_width;
@@ -465,7 +462,8 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
   // the heads that waves take: queries; keys and, token by token, values if they go to the cache
   const int heads = write_kv == 0 ? nq : (write_kv == 1 ? nq + 2 * nkv : nq + nkv);
   // a prompt portion's waves take four heads each; a few tokens' take one, spread over the machine
-  const int hpw = vec && num_tokens >= 256 ? 4 : 1;
+  // (as many as give each of a block's four waves its share of the heads, four at most)
+  const int hpw = vec && num_tokens >= 256 ? (heads >= 13 ? 4 : (heads + 3) / 4) : 1;
   int rows = rv_div_up(vec ? heads : (write_kv == 1 ? nq + 2 * nkv : nq + nkv), 4 * hpw);
   if (write_kv == 2) {
     RV_CHECK(slices == 0 && q_start && chunk_start && num_requests >= 1 && max_portion >= 1,
@@ -482,9 +480,11 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
       token_req, block_table, table_width, (TT*)k_pages, (TT*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv, V)
   if (vec) {
     if (dtype == RV_F32) {
-      if (hpw == 4) QKR_VEC_LAUNCH(float, 4); else QKR_VEC_LAUNCH(float, 1);
+      if (hpw == 4) QKR_VEC_LAUNCH(float, 4); else if (hpw == 3) QKR_VEC_LAUNCH(float, 3);
+      else if (hpw == 2) QKR_VEC_LAUNCH(float, 2); else QKR_VEC_LAUNCH(float, 1);
     } else if (dtype == RV_BF16) {
-      if (hpw == 4) QKR_VEC_LAUNCH(bf16_t, 4); else QKR_VEC_LAUNCH(bf16_t, 1);
+      if (hpw == 4) QKR_VEC_LAUNCH(bf16_t, 4); else if (hpw == 3) QKR_VEC_LAUNCH(bf16_t, 3);
+      else if (hpw == 2) QKR_VEC_LAUNCH(bf16_t, 2); else QKR_VEC_LAUNCH(bf16_t, 1);
     } else {
       return rv_fail("qk_norm_rope: unsupported dtype %d", dtype);
     }
