@@ -154,7 +154,9 @@ def time_decode(engine_parts, batch: int, context: int, steps: int, warmup: int)
     return elapsed / steps
 
 
-def time_prefill(engine_parts, length: int, repeats: int):
+def time_prefill(engine_parts, length: int, repeats: int, start: int = 0):
+    """A prompt portion of ``length`` tokens through the step function; with ``start`` the portion continues a
+    request that already holds ``start`` tokens (their keys and values random)."""
     torch, runner, sampler, SamplingParams, SplitMix64 = engine_parts
     vocab = runner.model.spec.vocab_size
     g = torch.Generator().manual_seed(2)
@@ -164,6 +166,8 @@ def time_prefill(engine_parts, length: int, repeats: int):
     for i in range(repeats + 1):
         rid = f"prefill-{i}"
         runner.add_request(rid)
+        if start > 0:
+            runner.cache.adopt_length_for_measurement(rid, start)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         logits = runner.step([(rid, prompt, [length - 1])])
@@ -318,6 +322,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers of the same size (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--prefill-at", type=int, default=0,
+                    help="the prompt portion continues a request that already holds this many tokens")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-probes", action="store_true", help="skip the measured peaks (read rate, library product)")
@@ -350,9 +356,9 @@ def main() -> int:
     max_batch = max(args.batch, 1 if args.no_points else 64)
     steps_total = args.steps + args.warmup + 8
     engine_cfg = EngineConfig(
-        dtype=args.dtype, page_size=16, max_model_len=args.context + steps_total,
+        dtype=args.dtype, page_size=16, max_model_len=max(args.context + steps_total, args.prefill_at + args.prefill_tokens),
         max_num_seqs=max_batch, max_num_batched_tokens=max(args.prefill_tokens, max_batch),
-        max_prefill_chunk=max(args.prefill_tokens, 1), max_cache_tokens=max_batch * (args.context + steps_total + 16),
+        max_prefill_chunk=max(args.prefill_tokens, 1), max_cache_tokens=max(max_batch * (args.context + steps_total + 16), args.prefill_at + args.prefill_tokens + 64),
         use_graphs=bool(args.graphs),
         **({} if args.steps_ahead is None else {"greedy_steps_ahead": args.steps_ahead}))
     log(f"building {args.layers}-layer model with random weights ({short})")
@@ -418,10 +424,19 @@ def main() -> int:
         result["roofline"]["frac_of_measured"] = round(achieved / peaks["hbm_read_GBs"], 4)
     if not args.no_prefill:
         T = args.prefill_tokens
-        psec, pmin = time_prefill(parts, T, repeats=5)
-        flops = T * layer_flops_per_token + attention_flops(cfg, 0, T) + head_flops_per_row
+        if args.prefill_at > 0:  # the cache's pages hold random keys and values, as for the decode points
+            gen = torch.Generator(device=runner.device)
+            gen.manual_seed(3)
+            for view in runner.storage.views:
+                if view is not None and hasattr(view, "k_pages"):
+                    view.k_pages.normal_(0.0, 1.0, generator=gen)
+                    view.v_pages.normal_(0.0, 1.0, generator=gen)
+        psec, pmin = time_prefill(parts, T, repeats=5, start=args.prefill_at)
+        flops = T * layer_flops_per_token + attention_flops(cfg, args.prefill_at, T) + head_flops_per_row
         result["prefill"] = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
                              "frac": round(flops / psec / PEAK_FLOPS[short], 4), "ms_min": round(pmin * 1e3, 3)}
+        if args.prefill_at > 0:
+            result["prefill"]["at"] = args.prefill_at
         if "gemm_bf16_TFLOPs" in peaks:
             result["prefill"]["measured_peak_TFLOPs"] = peaks["gemm_bf16_TFLOPs"]
             result["prefill"]["frac_of_measured"] = round(flops / psec / (peaks["gemm_bf16_TFLOPs"] * 1e12), 4)

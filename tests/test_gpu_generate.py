@@ -281,14 +281,18 @@ def test_eos_and_capacity_reasons(model_dirs):
     assert res.finish_reason == "capacity" and 0 < len(res.tokens) < 100
 
 
-def test_command_line(model_dirs, tmp_path):
+@pytest.mark.parametrize("how", ["module", "script"])
+def test_command_line(model_dirs, tmp_path, how):
+    """As ``python -m rvllm_amd.cli`` and as the script ``bin/rvllm-amd``, from another working folder."""
     prompts = tmp_path / "prompts.txt"
     prompts.write_text("1 2 3 4\n9 8 7\n")
     dump = tmp_path / "out.txt"
-    cmd = [sys.executable, "-m", "rvllm_amd.cli", "--model", str(model_dirs["A"]), "--dtype=float32",
+    start = [sys.executable, "-m", "rvllm_amd.cli"] if how == "module" else [str(tt.ROOT / "bin" / "rvllm-amd")]
+    cmd = [*start, "--model", str(model_dirs["A"]), "--dtype=float32",
            "--max-model-len", "64", "--max-num-seqs", "2", "--prompt-file", str(prompts), "--max-tokens", "5",
            "--dump", str(dump)]
-    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=str(tt.ROOT), timeout=300)
+    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=str(tt.ROOT if how == "module" else tmp_path),
+                          timeout=300)
     assert proc.returncode == 0, proc.stderr
     lines = [json.loads(l) for l in proc.stdout.strip().splitlines()]
     assert [l["completion_tokens"] for l in lines] == [5, 5] and lines[0]["finish_reason"] == "length"
