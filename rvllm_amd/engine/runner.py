@@ -31,6 +31,21 @@ from ..weights.loader import load_tensors, open_model_files, tensor_names
 from ..weights.random_init import random_tensors
 from .batch import BatchBuilder, Portion, StepBatch
 
+_frozen = False
+
+
+def _freeze_what_exists_once() -> None:
+    """What exists when the first engine of a process is built (the interpreter's modules, the libraries' objects)
+    lives as long as the process: taken out of the garbage collector's sight, so that a full collection between two
+    steps, which would walk all of it (some 100 ms with the libraries loaded here), has little to walk.  Once only:
+    what is frozen is never collected, and an engine built and dropped later must still be."""
+    global _frozen
+    if not _frozen:
+        _frozen = True
+        gc.collect()
+        gc.freeze()
+
+
 class ModelRunner:
     def __init__(self, model: DecoderModel, engine_config: EngineConfig):
         """``model`` has its weights bound already."""
@@ -66,11 +81,7 @@ class ModelRunner:
         self._graphs: collections.OrderedDict[tuple[int, int], tuple] = collections.OrderedDict()
         self._graph_pool = None
         self.graph_replays = 0
-        # What exists now (the interpreter's modules, the model) lives as long as the engine: taken out of the
-        # garbage collector's sight, so that a full collection between two steps, which would walk all of it
-        # (some 100 ms with the libraries loaded here), has almost nothing to walk.
-        gc.collect()
-        gc.freeze()
+        _freeze_what_exists_once()
 
     # ---- decode steps from captured graphs -------------------------------
     GRAPH_CONTEXT_BUCKET = 1024
