@@ -433,6 +433,111 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
   }
 }
 
+// Prompt portions in bf16 (thousands of tokens, the projection whole): a lane holds 8 neighbouring dimensions
+// (16 bytes), so a head of hd dimensions takes hd / 8 lanes (a power of two up to 32) and a wave works on 64 / (hd / 8)
+// heads at a time, `PASSES` such sets one after the other with all their reads asked for at once; the token's
+// cosines and sines, its place in the cache and the norm's weights are read once for all of them.  Sums and exchanges
+// stay inside a head's lanes.  A third of the memory instructions of the kernel above for the same bytes; the values
+// are written a page at a time by the extra rows of blocks, as there.
+#define QKP_PASSES 3
+__global__ void __launch_bounds__(256)
+qk_norm_rope_prompt_kernel(const uint16_t* __restrict__ qkv, uint16_t* __restrict__ q_out, const void* __restrict__ q_w,
+                           const void* __restrict__ k_w, int w_f32, float eps, float offset,
+                           const float* __restrict__ rope_cos, const float* __restrict__ rope_sin, int rot,
+                           const int* __restrict__ positions, const int* __restrict__ token_req,
+                           const int* __restrict__ block_table, int table_width, uint16_t* __restrict__ k_pages,
+                           uint16_t* __restrict__ v_pages, int page_size, int num_pages, int nq, int nkv, int hd,
+                           int write_kv, int num_tokens, int waves_per_token, int head_rows, ValuePages V) {
+  if ((int)blockIdx.y >= head_rows) {  // the rows of the grid beyond the heads write values a page at a time
+    v_write_page<bf16_t>((long long)(blockIdx.y - head_rows) * gridDim.x + blockIdx.x, V, (const bf16_t*)qkv,
+                         (bf16_t*)v_pages, block_table, table_width, page_size, num_pages, nq, nkv, hd);
+    return;
+  }
+  const int lane = threadIdx.x & 63;
+  const int wave_id = (blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int t = wave_id / waves_per_token;
+  if (t >= num_tokens) return;  // the whole wave
+  const int lph = hd >> 3;                    // lanes a head
+  const int hpp = 64 / lph;                   // heads a pass
+  const int hl = lane / lph;                  // this lane's head within a pass
+  const int l = lane - hl * lph;              // this lane within its head
+  const int d0 = l * 8;
+  const int heads = write_kv != 0 ? nq + nkv : nq;  // queries, and keys if they go to the cache
+  const int total_heads = nq + 2 * nkv;
+  const int head_first = (wave_id - t * waves_per_token) * QKP_PASSES * hpp + hl;
+  const size_t row = (size_t)t * total_heads * hd;
+
+  uint4 raw[QKP_PASSES];
+#pragma unroll
+  for (int p = 0; p < QKP_PASSES; ++p) {
+    const int head = head_first + p * hpp;
+    raw[p] = *(const uint4*)(qkv + row + (size_t)(head < heads ? head : heads - 1) * hd + d0);  // past the end: dropped
+  }
+  const int rot_half = rot >> 1;
+  const bool first_half = l < (lph >> 1);
+  const int pd0 = first_half ? d0 : d0 - (hd >> 1);  // the pairs' index
+  const bool turns = pd0 < rot_half;
+  float c[8] = {1, 1, 1, 1, 1, 1, 1, 1}, sn[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (rot_half > 0) {
+    const float* pc = rope_cos + (size_t)t * rot_half + (turns ? pd0 : 0);
+    const float* pn = rope_sin + (size_t)t * rot_half + (turns ? pd0 : 0);
+    const float4 c0 = *(const float4*)pc, c1 = *(const float4*)(pc + 4), n0 = *(const float4*)pn, n1 = *(const float4*)(pn + 4);
+    c[0] = c0.x, c[1] = c0.y, c[2] = c0.z, c[3] = c0.w, c[4] = c1.x, c[5] = c1.y, c[6] = c1.z, c[7] = c1.w;
+    sn[0] = n0.x, sn[1] = n0.y, sn[2] = n0.z, sn[3] = n0.w, sn[4] = n1.x, sn[5] = n1.y, sn[6] = n1.z, sn[7] = n1.w;
+  }
+  float g_q[8], g_k[8];
+  if (q_w != nullptr) {
+    rv_load_w_vec<8>(q_w, w_f32, d0, g_q);
+    rv_load_w_vec<8>(k_w, w_f32, d0, g_k);
+  }
+  int page = -1, slot = 0;
+  if (write_kv != 0) {
+    const int pos = positions[t];
+    const int logical = pos / page_size;
+    slot = pos - logical * page_size;
+    if (logical < table_width) page = block_table[(size_t)token_req[t] * table_width + logical];
+    if (page >= num_pages) page = -1;
+  }
+#pragma unroll
+  for (int p = 0; p < QKP_PASSES; ++p) {
+    const int head = head_first + p * hpp;
+    const bool there = head < heads;  // lanes of a head decide alike; the exchanges below take every lane
+    const bool is_q = head < nq;
+    float x[8];
+    {
+      const uint32_t u[4] = {raw[p].x, raw[p].y, raw[p].z, raw[p].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[2 * i] = __uint_as_float(u[i] << 16), x[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+    }
+    if (q_w != nullptr) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+      for (int off = lph >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, RV_WAVE);  // over the head's lanes
+      const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = x[i] * inv * (offset + (is_q ? g_q[i] : g_k[i]));
+    }
+    if (rot_half > 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float other = __shfl_xor(x[i], lph >> 1, RV_WAVE);  // the other half of the pair
+        if (turns) x[i] = first_half ? x[i] * c[i] - other * sn[i] : x[i] * c[i] + other * sn[i];
+      }
+    }
+    if (!there) continue;
+    uint16_t* dst;
+    if (is_q) {
+      dst = q_out + ((size_t)t * nq + head) * hd;
+    } else {
+      if (page < 0) continue;
+      dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
+    }
+    *(uint4*)(dst + d0) = make_uint4(rv_pack_bf16x2(x[0], x[1]), rv_pack_bf16x2(x[2], x[3]), rv_pack_bf16x2(x[4], x[5]),
+                                     rv_pack_bf16x2(x[6], x[7]));
+  }
+}
+
 // `slices` 0: qkv holds T values [tokens, (nq + 2 nkv) * hd]; otherwise 32-bit
 // partial sums [slices][tokens][...], slice_stride elements apart.
 extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int slices, long long slice_stride,
@@ -472,6 +577,26 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
     const long long units = (long long)V.pages_per_request * nkv * num_requests;
     rows += (int)((units + num_tokens - 1) / num_tokens);
     RV_CHECK(rows <= 65535, "qk_norm_rope: too many pages of values for one launch");
+  }
+  // prompt portions in bf16 whose values go by pages: sixteen bytes a lane, several heads a wave at a time
+  const int lph = hd / 8;
+  if (write_kv == 2 && dtype == RV_BF16 && slices == 0 && hd % 8 == 0 && lph >= 2 && lph <= 32 && (lph & (lph - 1)) == 0 &&
+      rot % 16 == 0 && num_tokens >= 256 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)q_out % 16) == 0) {
+    const int heads_kq = nq + nkv;
+    const int per_wave = QKP_PASSES * (64 / lph);
+    const int waves_per_token = rv_div_up(heads_kq, per_wave);
+    const long long blocks = rv_div_up((long long)num_tokens * waves_per_token, 4);
+    const int gx = num_tokens;  // the page writer's rows count their blocks by this width
+    const int head_rows = rv_div_up(blocks, gx);
+    const long long units = (long long)V.pages_per_request * nkv * num_requests;
+    const int page_rows = (int)((units + gx - 1) / gx);
+    RV_CHECK(head_rows + page_rows <= 65535, "qk_norm_rope: too many blocks for one launch");
+    qk_norm_rope_prompt_kernel<<<dim3(gx, head_rows + page_rows), dim3(256), 0, stream>>>(
+        (const uint16_t*)qkv, (uint16_t*)q_out, q_w, k_w, w_f32, eps, offset, rope_cos, rope_sin, rot, positions, token_req,
+        block_table, table_width, (uint16_t*)k_pages, (uint16_t*)v_pages, page_size, num_pages, nq, nkv, hd, write_kv,
+        num_tokens, waves_per_token, head_rows, V);
+    RV_LAUNCH_CHECK("qk_norm_rope_prompt");
+    return 0;
   }
   dim3 grid(num_tokens, rows), block(4 * RV_WAVE);
 #define QKR_VEC_LAUNCH(TT, HPW)                                                                                        \

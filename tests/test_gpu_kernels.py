@@ -372,6 +372,51 @@ def test_values_written_a_page_at_a_time(dtype, page_size, longest):
             t += 1
 
 
+@pytest.mark.parametrize("nq,nkv,hd,rot", [(8, 4, 256, 256), (5, 1, 128, 64), (7, 3, 64, 64), (3, 2, 16, 16), (6, 2, 32, 0),
+                                          (13, 5, 64, 32), (1, 1, 256, 128)])
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_qk_norm_rope_of_a_prompt_portion(nq, nkv, hd, rot, page_size):
+    """Some hundred tokens in bf16 with the values written by pages take the kernel that holds eight dimensions a
+    lane and several heads a wave: heads that fill a wave's passes and heads that do not, a rotation of the whole
+    head, of a part and none, portions that begin inside pages.  Against the plain formulas, and against the kernel
+    that takes a head a wave."""
+    dtype = torch.bfloat16
+    portions = [(5, 290), (64, 32), (0, 1), (31, 2), (100, 16)]
+    case = Case(portions, nq, nkv, hd, page_size, dtype, 23)
+    T = case.q.shape[0]
+    g = torch.Generator().manual_seed(24)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd, generator=g).to(dtype)
+    qw = (torch.randn(hd, generator=g) * 0.1).to(dtype)
+    kw = (torch.randn(hd, generator=g) * 0.1).to(dtype)
+    inv_freq = (10000.0 ** (-2.0 * torch.arange(rot // 2, dtype=torch.float64) / hd) / 4.0).float()
+    rope = ops.rope_table(dev(inv_freq), case.step.positions, T) if rot else None
+    results = []
+    for by_page in (False, True):
+        kp, vp = to_cache(torch.zeros_like(case.k_log), torch.zeros_like(case.v_log))
+        q_out = torch.full((T, nq * hd), float("nan"), dtype=dtype, device=DEV)
+        ops.qk_norm_rope_kv_write(dev(qkv), q_out, dev(qw), dev(kw), 1e-5, 1.0, rope, rot, case.step.positions,
+                                  case.step.token_req, dev(case.table), kp, vp, nq, nkv, hd,
+                                  values_by_page=case.step if by_page else None)
+        results.append((q_out.cpu(), kp.cpu(), vp.cpu()))
+    # the values are copied, so they are the same bits; the sums of squares are added up in another order
+    assert torch.equal(results[0][2].view(torch.int16), results[1][2].view(torch.int16))
+    for a, b in zip(results[0][:2], results[1][:2]):
+        assert torch.allclose(a.float(), b.float(), **tol(dtype))
+    q, k, _ = qkv.double().split([nq * hd, nkv * hd, nkv * hd], dim=1)
+    q = P.rmsnorm(q.view(T, nq, hd), qw.double(), 1e-5)
+    k = P.rmsnorm(k.view(T, nkv, hd), kw.double(), 1e-5)
+    if rot:
+        full = torch.zeros(hd // 2, dtype=torch.float64)
+        full[: rot // 2] = inv_freq.double()
+        q, k = P.rope(q, case.positions, full), P.rope(k, case.positions, full)
+    assert torch.allclose(results[1][0].float().view(T, nq, hd), q.float(), **tol(dtype))
+    kp, _ = from_cache(results[1][1].to(DEV), results[1][2].to(DEV))
+    for t in range(T):
+        b, pos = int(case.token_req[t]), int(case.positions[t])
+        page = int(case.table[b, pos // page_size])
+        assert torch.allclose(kp[page, pos % page_size].cpu().float(), k[t].float(), **tol(dtype)), t
+
+
 def test_rope_table_against_64_bit_angles():
     """cos and sin of float32(position) * inv_freq, positions up to a long context, against 64-bit
     functions of the same 32-bit angle."""
