@@ -8,8 +8,11 @@ but its kernels' interface already describes several portions at once by
 this batch is that description, extended by the request of every token so that
 token-wise kernels need no search.
 
-All index arrays travel to the GPU as one packed int32 buffer with one copy
-(the reference's packed metadata buffer: v3/crates/rvllm-metadata/src/layout.rs:19-78).
+All index arrays lie in one packed int32 buffer (the reference's packed
+metadata buffer: v3/crates/rvllm-metadata/src/layout.rs:19-78).  The arrays by
+token and by request travel to the GPU with one copy; of each block table, as
+wide as the longest context the engine allows, only the step's requests by the
+pages of the longest of them travel, as one strided copy.
 """
 
 from __future__ import annotations
@@ -19,6 +22,8 @@ from typing import Optional, Sequence
 
 import numpy as np
 import torch
+
+from ..kernels import ops
 
 
 @dataclasses.dataclass
@@ -87,6 +92,7 @@ class BatchLayout:
         add("chunk_start", max_requests)
         add("context_len", max_requests)
         add("state_slot", max_requests)
+        self.tables_from = off  # what lies before is copied whole each step
         for name, width in self.table_widths.items():
             add("bt:" + name, max_requests * width)
         self.total = off
@@ -107,6 +113,11 @@ class BatchBuilder:
         self.host = self._hosts[0]
         self.host_np = self.host.numpy()
         self.dev = torch.zeros(self.layout.total, dtype=torch.int32, device=self.device)
+        self.dev[self.layout.tables_from :] = -1  # no page anywhere, until a step says otherwise
+
+    def _table(self, buffer: torch.Tensor, name: str) -> torch.Tensor:
+        off, cap = self.layout.offsets["bt:" + name]
+        return buffer[off : off + cap].view(self.layout.max_requests, self.layout.table_widths[name])
 
     def _view(self, name: str, n: Optional[int] = None) -> torch.Tensor:
         off, cap = self.layout.offsets[name]
@@ -162,14 +173,16 @@ class BatchBuilder:
         rows[:r] = wanted
         max_portion = max(1, int(lens.max())) if B else 1
         max_context = max(1, int((starts + lens).max())) if B else 1
+        used = {}  # group -> entries of the step's longest table: what the step's kernels can ask for
         for name, width in lay.table_widths.items():
             off, _ = lay.offsets["bt:" + name]
             dst = self.host_np[off : off + B * width]
-            dst.fill(-1)
             held = [np.asarray(row, dtype=np.int32) for row in tables[name]]
             counts = np.fromiter((len(row) for row in held), dtype=np.int64, count=B)
             if B and counts.max() > width:
                 raise ValueError(f"block table of group {name} has {int(counts.max())} entries, width is {width}")
+            used[name] = int(counts.max()) if B else 0
+            dst.reshape(B, width)[:, : used[name]] = -1
             total = int(counts.sum())
             if total:
                 # entry j of row b goes to b * width + j
@@ -180,13 +193,18 @@ class BatchBuilder:
                 where = np.repeat(np.arange(B, dtype=np.int64) * width - row_first, counts)
                 where += np.arange(total, dtype=np.int64)
                 dst[where] = np.concatenate(held)
-        self.dev.copy_(self.host, non_blocking=True)
+        self.dev[: lay.tables_from].copy_(self.host[: lay.tables_from], non_blocking=True)
+        tables_dev = {}
+        for name in lay.table_widths:
+            tables_dev[name] = self._table(self.dev, name)
+            # Rows beyond the step's requests and entries beyond its longest table keep what earlier steps left:
+            # no kernel looks there, since a request's keys end with its own context.
+            if event is not None:
+                ops.copy_rows_to_device(tables_dev[name], self._table(self.host, name), B, used[name])
+            else:
+                tables_dev[name][:B, : used[name]] = self._table(self.host, name)[:B, : used[name]]
         if event is not None:
             event.record()
-        tables_dev = {}
-        for name, width in lay.table_widths.items():
-            off, _ = lay.offsets["bt:" + name]
-            tables_dev[name] = self.dev[off : off + lay.max_requests * width].view(lay.max_requests, width)
         return StepBatch(
             num_tokens=T,
             num_requests=B,

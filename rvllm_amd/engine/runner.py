@@ -107,8 +107,18 @@ class ModelRunner:
             return None
         if not self.model.capturable:  # a part waits for the device or launches by its data
             return None
-        bucket = -(-max_context // self.GRAPH_CONTEXT_BUCKET) * self.GRAPH_CONTEXT_BUCKET
-        return num_requests, bucket
+        return num_requests, self.context_bucket(max_context)
+
+    @classmethod
+    def context_bucket(cls, max_context: int) -> int:
+        """The upper end of the bucket of contexts that one captured graph serves.  Buckets are
+        GRAPH_CONTEXT_BUCKET wide up to sixteen of them and then double with the context, so that a graph's
+        plan is made for at most an eighth more keys than there are, and a batch that decodes from a long
+        context to a longer one records a graph every few thousand steps rather than every thousand."""
+        width = cls.GRAPH_CONTEXT_BUCKET
+        while max_context > 16 * width:
+            width *= 2
+        return -(-max_context // width) * width
 
     def _forward(self, batch: StepBatch) -> torch.Tensor:
         key = self._graph_key(batch)
@@ -122,8 +132,18 @@ class ModelRunner:
             shaped = dataclasses.replace(batch, max_context=key[1], shared={})  # nothing made outside the recording
             graph = torch.cuda.CUDAGraph()
             torch.cuda.synchronize()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                static_logits = self.model.forward(shaped, self.storage.views)
+            # No garbage collection while the stream records: an engine dropped earlier in the process may lie
+            # in a cycle with its graphs and their memory, and freeing those is not allowed during a recording
+            # (the process aborts).  What is garbage now goes before; the collector rests until the recording ends.
+            gc.collect()
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph, pool=self._graph_pool):
+                    static_logits = self.model.forward(shaped, self.storage.views)
+            finally:
+                if collecting:
+                    gc.enable()
             if self._graph_pool is None:
                 self._graph_pool = graph.pool()
             self._graphs[key] = (graph, static_logits)

@@ -619,6 +619,21 @@ def advance_decode(step, chosen: torch.Tensor) -> None:
                                        _ptr(step.chunk_start), _ptr(step.context_len), _c_int(n)))
 
 
+def copy_rows_to_device(dst: torch.Tensor, src: torch.Tensor, rows: int, cols: int) -> None:
+    """``dst[:rows, :cols] = src[:rows, :cols]`` from a pinned host matrix to a device matrix of the same element
+    size as one strided copy in the current stream's order (rows far apart, as a step's block tables are: only
+    the pages that the step's requests hold travel)."""
+    _gpu(dst)
+    _need(not src.is_cuda and src.is_pinned(), "copy_rows: the source must be pinned host memory")
+    _need(dst.dim() == 2 and src.dim() == 2 and dst.element_size() == src.element_size()
+          and dst.stride(1) == 1 and src.stride(1) == 1, "copy_rows: two matrices with rows of the same elements expected")
+    _need(0 <= rows <= min(dst.shape[0], src.shape[0]) and 0 <= cols <= min(dst.shape[1], src.shape[1]),
+          f"copy_rows: {rows} x {cols} does not fit {tuple(src.shape)} -> {tuple(dst.shape)}")
+    e = dst.element_size()
+    _check(library().rv_copy_rows_to_device(_stream(), _ptr(dst), _c_ll(dst.stride(0) * e), _ptr(src),
+                                            _c_ll(src.stride(0) * e), _c_ll(cols * e), _c_ll(rows)))
+
+
 def topk_select(logits: torch.Tensor, k: int, inv_temp: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """The k largest logits of every row, times 1/T, with their ids (unordered)."""
     _gpu(logits, inv_temp)

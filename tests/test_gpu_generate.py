@@ -190,6 +190,32 @@ def test_a_graph_dropped_for_room_is_recorded_again(model_dirs, plain_models):
     assert replays == [0, 1, 1, 1, 1] * 3  # the first step of each run of a shape is eager
 
 
+def test_the_garbage_collector_rests_while_a_step_is_recorded(model_dirs):
+    """An engine that was dropped may lie in a cycle with its graphs; were it collected while another step is being
+    recorded, its memory would be freed during the recording, which the runtime does not allow.  So what is garbage
+    goes before the recording and the collector is off during it, and as it was afterwards."""
+    import gc
+
+    cfg = EngineConfig(dtype="bfloat16", max_model_len=256, max_num_seqs=2, max_num_batched_tokens=256,
+                       max_prefill_chunk=256, max_cache_tokens=512, use_graphs=True)
+    runner = LLMEngine.from_model_dir(model_dirs["A"], cfg).runner
+    seen = []
+    forward = runner.model.forward
+
+    def watched(batch, views):
+        seen.append((torch.cuda.is_current_stream_capturing(), gc.isenabled()))
+        return forward(batch, views)
+
+    runner.model.forward = watched
+    runner.add_request("a")
+    runner.step([("a", [1, 2, 3], [2])])
+    assert gc.isenabled()
+    for token in (4, 5, 6):
+        runner.step([("a", [token], [0])])
+    # the prompt, the first decoded token run as it comes and then recorded; the rest are replays
+    assert seen == [(False, True), (False, True), (True, False)] and gc.isenabled() and runner.graph_replays == 2
+
+
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_several_greedy_steps_in_a_row_choose_what_single_steps_choose(model_dirs, name):
     """``decode_greedy`` hands each request's arg-max token to its next step on the device.  Against a twin runner
