@@ -106,9 +106,11 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   constexpr int PIECES = MT * 16 * (SK_KC / 8);  // 16-byte pieces in a chunk
   // a thread holds at most PIECES / 256 pieces (blocks have at least 4 waves)
   constexpr int MAX_REGS = (PIECES + 255) / 256;
-  uint4 staged[MAX_REGS];
+  // One set of registers per chunk of a pass: a set that is loaded at two places of the loop gets copied by the
+  // compiler right after the second load, and the copy waits for every read asked for before it, the ring's too.
+  uint4 staged_sets[UNROLL][MAX_REGS];
   const int last_k = kend - 8;  // the last 16-byte piece of this slice (slices are multiples of 8 long)
-  auto stage_load = [&](int c) {
+  auto stage_load = [&](int c, uint4 (&staged)[MAX_REGS]) {
 #pragma unroll
     for (int n = 0; n < MAX_REGS; ++n) {
       int p = tid + n * (int)blockDim.x;
@@ -120,7 +122,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
       staged[n] = *(const uint4*)(x + (size_t)m * ldx + k);
     }
   };
-  auto stage_store = [&](int c, int buf) {
+  auto stage_store = [&](int c, int buf, uint4 (&staged)[MAX_REGS]) {
 #pragma unroll
     for (int n = 0; n < MAX_REGS; ++n) {
       int p = tid + n * (int)blockDim.x;
@@ -167,43 +169,57 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   // The first chunk of x and the whole ring are requested together.  The order
   // (x, then the ring's places in turn) is the one every pass of the loop below
   // leaves behind, so the compiler's count of reads in flight is exact there.
-  stage_load(0);
+  stage_load(0, staged_sets[0]);
   asm volatile("" ::: "memory");
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
     load_w(d * 128, ring[d]);
     asm volatile("" ::: "memory");
   }
-  stage_store(0, 0);
+  stage_store(0, 0, staged_sets[0]);
   __syncthreads();
 
   int c = 0;
   do {  // a slice has at least one chunk; a loop that may run zero times lets the first reads sink below the barrier
+    // the x of the chunks after this pass's: asked for here, all of it, before the ring's reads, so that waiting
+    // for it leaves those in flight; in flight while this pass's chunks are multiplied
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) stage_load(c + u + 1, staged_sets[u]);
+    asm volatile("" ::: "memory");
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       // chunk c + u: its x lies in buffer `buf`, its W in the ring's places u * CH .. u * CH + CH - 1.  A chunk
       // past the slice's end (an odd number of chunks, two a pass) meets zeros of x.
       const int cc = c + u;
       const int buf = UNROLL == 1 ? (c & 1) : (u & 1);
-      stage_load(cc + 1);  // in flight while this chunk is multiplied
-      asm volatile("" ::: "memory");  // issued before the ring's reads, so that waiting for it leaves those in flight
 #pragma unroll
       for (int st = 0; st < CH; ++st) {
         const int d = u * CH + st;
+        // The operands from x of several products are asked for before the first of them: a read from LDS takes
+        // some hundred cycles, and one or two in flight make sixteen of them a step longer than the step's share
+        // of the memory's time.  A whole step's at once up to 32 rows of x; beyond, half a step's (registers).
+        constexpr int JG = MT <= 2 ? 4 : 2;  // 128-column quarters whose operands are in flight together
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int col = st * 128 + j * 32 + kb * 8;
+        for (int j0 = 0; j0 < 4; j0 += JG) {
+          SkFrag b[JG][MT];
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            SkFrag b;
-            b.u4 = *(const uint4*)(&xs[buf][mt * 16 + r16][col]);
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[d][j].v, b.v, acc[mt], 0, 0, 0);
+          for (int j = 0; j < JG; ++j) {
+            const int col = st * 128 + (j0 + j) * 32 + kb * 8;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) b[j][mt].u4 = *(const uint4*)(&xs[buf][mt * 16 + r16][col]);
+          }
+          __builtin_amdgcn_sched_barrier(0);  // or the compiler puts each read back before its product
+#pragma unroll
+          for (int j = 0; j < JG; ++j) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[d][j0 + j].v, b[j][mt].v, acc[mt], 0, 0, 0);
           }
         }
         load_w((cc + UNROLL) * SK_KC + st * 128, ring[d]);  // the same place of the ring, a ring's length on
         asm volatile("" ::: "memory");                     // here, and not gathered at the chunk's end
       }
-      stage_store(cc + 1, buf ^ 1);  // that buffer was last read in chunk cc - 1, before the barrier below
+      stage_store(cc + 1, buf ^ 1, staged_sets[u]);  // that buffer was last read in chunk cc - 1, before the barrier below
       __syncthreads();
     }
     c += UNROLL;
