@@ -307,6 +307,64 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ branch, int slices, 
   }
 }
 
+// The same for many rows in bf16 (a prompt portion): a wave takes a whole row, eight values a lane and turn, so
+// both sums are exchanges inside the wave and no barrier stands between a row's reads and its writes.  The
+// arithmetic is the block kernel's, value by value; only the order in which a row's squares are added differs.
+template <int E>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_rows_kernel(const uint16_t* __restrict__ branch, const void* __restrict__ w_post, int w_post_f32,
+                        uint16_t* __restrict__ residual, const void* __restrict__ w_next, int w_next_f32,
+                        uint16_t* __restrict__ next, int rows, int width, float eps, float offset, float eps_next,
+                        float offset_next) {
+  const int lane = threadIdx.x & (RV_WAVE - 1);
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;  // the whole wave
+  const size_t row0 = (size_t)row * width;
+  float val[E][8], res[E][8], g_post[E][8], g_next[E][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = (e * RV_WAVE + lane) * 8;
+    if (i < width) {
+      row_load<bf16_t, 8>((const bf16_t*)branch + row0 + i, val[e]);
+      row_load<bf16_t, 8>((const bf16_t*)residual + row0 + i, res[e]);
+      row_load_w<8>(w_post, w_post_f32, i, g_post[e]);
+      if (next != nullptr) row_load_w<8>(w_next, w_next_f32, i, g_next[e]);
+#pragma unroll
+      for (int v = 0; v < 8; ++v) ss += val[e][v] * val[e][v];
+    }
+  }
+  ss = rv_wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = (e * RV_WAVE + lane) * 8;
+    if (i < width) {
+#pragma unroll
+      for (int v = 0; v < 8; ++v) {
+        val[e][v] = rv_round_to<bf16_t>(res[e][v] + val[e][v] * inv * (offset + g_post[e][v]));
+        ss2 += val[e][v] * val[e][v];
+      }
+      row_store<bf16_t, 8>((bf16_t*)residual + row0 + i, val[e]);
+    }
+  }
+  if (next == nullptr) return;
+  ss2 = rv_wave_sum(ss2);
+  const float inv2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = (e * RV_WAVE + lane) * 8;
+    if (i < width) {
+#pragma unroll
+      for (int v = 0; v < 8; ++v) val[e][v] = val[e][v] * inv2 * (offset_next + g_next[e][v]);
+      row_store<bf16_t, 8>((bf16_t*)next + row0 + i, val[e]);
+    }
+  }
+}
+#define ADD_RMSNORM_ROWS_MIN 256   // from this many rows on a wave takes a row
+#define ADD_RMSNORM_ROWS_MAX_E 6   // turns of 512 values a wave takes at most (its registers)
+
 // `slices` 0: branch holds T values [rows, width].  Otherwise branch holds
 // 32-bit partial sums [slices][rows][width] (slice_stride elements apart).
 extern "C" int rv_add_rmsnorm(hipStream_t stream, const void* branch, int slices, long long slice_stride,
@@ -317,6 +375,25 @@ extern "C" int rv_add_rmsnorm(hipStream_t stream, const void* branch, int slices
   RV_CHECK((w_next == nullptr) == (next == nullptr), "add_rmsnorm: next norm needs both weight and output");
   RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= (long long)rows * width), "add_rmsnorm: bad partial sums");
   if (rows == 0) return 0;
+  const int turns = rv_div_up(width, 8 * RV_WAVE);
+  if (dtype == RV_BF16 && slices == 0 && rows >= ADD_RMSNORM_ROWS_MIN && width % 8 == 0 &&
+      turns <= ADD_RMSNORM_ROWS_MAX_E) {
+#define RV_ARR(E)                                                                                                  \
+  add_rmsnorm_rows_kernel<E><<<dim3(rv_div_up(rows, 4)), dim3(256), 0, stream>>>(                                 \
+      (const uint16_t*)branch, w_post, w_post_f32, (uint16_t*)residual, w_next, w_next_f32, (uint16_t*)next, rows, \
+      width, eps, offset, eps_next, offset_next)
+    switch (turns) {
+      case 1: RV_ARR(1); break;
+      case 2: RV_ARR(2); break;
+      case 3: RV_ARR(3); break;
+      case 4: RV_ARR(4); break;
+      case 5: RV_ARR(5); break;
+      default: RV_ARR(6); break;
+    }
+#undef RV_ARR
+    RV_LAUNCH_CHECK("add_rmsnorm_rows");
+    return 0;
+  }
   dim3 grid(rows);
   if (dtype == RV_F32)
     ROW_DISPATCH(add_rmsnorm_kernel, float, width, grid, stream, branch, slices, slice_stride, w_post, w_post_f32,

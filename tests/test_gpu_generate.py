@@ -220,7 +220,8 @@ def test_the_garbage_collector_rests_while_a_step_is_recorded(model_dirs):
 def test_several_greedy_steps_in_a_row_choose_what_single_steps_choose(model_dirs, name):
     """``decode_greedy`` hands each request's arg-max token to its next step on the device.  Against a twin runner
     that takes one step at a time: the same tokens, over page edges, with requests of different lengths; one step
-    only while the shape has no graph yet, and no step past the end of the graph's bucket of contexts."""
+    only while the shape has no graph yet, and no step past the end of the graph's bucket of contexts.  (The engine
+    against the engine: what a single step computes is held to the plain model by the replay tests.)"""
     common = dict(dtype="bfloat16", max_model_len=1100, max_num_seqs=4, max_num_batched_tokens=1100,
                   max_prefill_chunk=1100, max_cache_tokens=3400, use_graphs=True)
     one = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(**common)).runner
@@ -256,7 +257,8 @@ def test_several_greedy_steps_in_a_row_choose_what_single_steps_choose(model_dir
 def test_greedy_steps_ahead_change_no_token(model_dirs, name):
     """Several greedy decode steps from one plan against one plan a step: the same tokens and reasons for requests
     that end at different lengths, one of them at an end id met on the way, with a request that samples among them
-    (then every step is planned by itself), and with so few pages that requests are set back."""
+    (then every step is planned by itself), and with so few pages that requests are set back.  (The engine
+    against the engine: what a single step computes is held to the plain model by the replay tests.)"""
     def run(ahead, tight, places=4):
         engine = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(
             dtype="bfloat16", max_model_len=200, max_num_seqs=places, max_num_batched_tokens=64, max_prefill_chunk=64,

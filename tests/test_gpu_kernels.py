@@ -86,6 +86,34 @@ def test_add_rmsnorm_with_and_without_the_next_norm(dtype, width):
     assert torch.allclose(nxt.cpu().float(), want_next.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("width", [96, 1000, 2560, 3072, 5376])
+@pytest.mark.parametrize("with_next", [True, False])
+def test_add_rmsnorm_of_many_rows(width, with_next):
+    """From some hundred rows on a wave takes a whole row (widths up to 3072; wider rows stay with the kernel
+    that gives a row to a block): a width that leaves most lanes without values, one that ends inside a turn
+    of the wave, whole turns, and rows that do not fill the last block."""
+    rows = 301
+    g = torch.Generator().manual_seed(33)
+    branch = (torch.randn(rows, width, generator=g) * 2).bfloat16()
+    res = torch.randn(rows, width, generator=g).bfloat16()
+    w1 = (torch.randn(width, generator=g) * 0.1).bfloat16()
+    w2 = (torch.randn(width, generator=g) * 0.1).bfloat16()
+    r = dev(res.clone())
+    nxt = ops.add_rmsnorm(dev(branch), dev(w1), 1e-6, 1.0, r, *((dev(w2), 1e-5, 1.0) if with_next else ()))
+    want_res = (res.double() + P.rmsnorm(branch.double(), w1.double(), 1e-6)).bfloat16()
+    assert torch.allclose(r.cpu().float(), want_res.float(), **tol(torch.bfloat16))
+    # a few rows at a time take the other kernel: the same values up to the order of a row's sum of squares
+    few = dev(res[:7].clone())
+    few_next = ops.add_rmsnorm(dev(branch[:7]), dev(w1), 1e-6, 1.0, few, *((dev(w2), 1e-5, 1.0) if with_next else ()))
+    assert torch.allclose(few.float(), r[:7].float(), rtol=1e-2, atol=1e-2)
+    if with_next:
+        want_next = P.rmsnorm(r.cpu().double(), w2.double(), 1e-5)  # of the residual as stored
+        assert torch.allclose(nxt.cpu().float(), want_next.float(), **tol(torch.bfloat16))
+        assert torch.allclose(few_next.float(), nxt[:7].float(), rtol=1e-2, atol=1e-2)
+    else:
+        assert nxt is None
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gated_act(dtype):
     g = torch.Generator().manual_seed(4)
