@@ -73,6 +73,27 @@ __device__ __forceinline__ void sk_store1<uint16_t>(uint16_t* p, float a) {
 // for it would read them): a kernel and a pass over memory less, at no cost.
 // A sliced product stores its partial sums as for ACT < 0.
 // TILED: W is stored in tiles (see rv_tile_weight); ldw is then unused.
+// A copy of 16 bytes a lane from memory straight into LDS: lane l's land at `to` + 16 l (`to` the same in all
+// lanes).  Written as an instruction of its own, so the compiler knows of no read from memory and of no write
+// to LDS: the wave that issues these issues no other reads from memory and counts them itself (sk_wait_copies).
+__device__ __forceinline__ void sk_copy16_to_lds(const void* from, const uint16_t* to) {
+  const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint16_t*)to;
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(from), "s"(at) : "memory", "m0");
+}
+// Waits until at most N of this wave's reads from memory are on their way (they arrive in the order of asking).
+template <int N>
+__device__ __forceinline__ void sk_wait_copies() {
+  static_assert(N >= 0 && N < 64, "the counter has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));  // vmcnt(N), nothing else
+  asm volatile("" ::: "memory");
+}
+__device__ const uint4 sk_zeros16 = {0u, 0u, 0u, 0u};  // what a copy reads where x has nothing
+
+// Beyond 32 rows of x a block has one wave more, which owns no rows of W and only brings x in (SK_BRINGERS_OF):
+// x is then as many bytes as W, and a wave that asks for both waits for its x behind the W it asked for earlier
+// (reads come back in the order of asking), with the barrier that follows, for the W of the whole next chunk and of
+// every wave of the block, which takes a quarter off the ring's depth.  The wave that brings x asks for nothing else.
+#define SK_BRINGERS_OF(MT) ((MT) >= 3 ? 3 : 0)
 template <int MT, typename TC, int ACT = -1, bool TILED = false>
 __global__ void __launch_bounds__(SK_MAX_WAVES * 64)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, TC* __restrict__ out,
@@ -83,14 +104,21 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   constexpr int UNROLL = DEPTH / CH;         // chunks a pass of the main loop takes
   constexpr int SK_KC = CH * 128;
   constexpr int SK_ROW = SK_KC + 8;
-  __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][SK_ROW];
+  // With waves that only bring x in, three buffers take turns: a chunk's x is on its way into one while the
+  // chunk before it is multiplied from another and the third still holds the one before that.  A copy fills
+  // 64 pieces of 16 bytes at a time, so a buffer has room behind its last row for the last copy's overhang.
+  constexpr int BUFS = SK_BRINGERS_OF(MT) > 0 ? 3 : 2;
+  constexpr int ROWS_ROOM = SK_BRINGERS_OF(MT) > 0 ? MT * 16 + 2 : MT * 16;
+  __shared__ __attribute__((aligned(16))) uint16_t xs[BUFS][ROWS_ROOM][SK_ROW];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int waves = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in all lanes, and known to be
+  constexpr int BRINGERS = SK_BRINGERS_OF(MT);
+  const int waves = (int)(blockDim.x >> 6) - BRINGERS;  // the waves that own rows of W
+  const bool brings_x = BRINGERS > 0 && wave >= waves;
   const int r16 = lane & 15;
   const int kb = lane >> 4;
-  const int n0 = (blockIdx.x * waves + wave) * 16;
+  const int n0 = (blockIdx.x * waves + (brings_x ? 0 : wave)) * 16;
   const bool wave_has_rows = n0 < N;
   const int row = n0 + r16 < N ? n0 + r16 : N - 1;
   const int kbeg = blockIdx.y * slice_len;
@@ -105,7 +133,9 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   // staging: the block copies x[0 : MT*16, chunk] into LDS, 16 bytes a thread and turn
   constexpr int PIECES = MT * 16 * (SK_KC / 8);  // 16-byte pieces in a chunk
   // a thread holds at most PIECES / 256 pieces (blocks have at least 4 waves)
-  constexpr int MAX_REGS = (PIECES + 255) / 256;
+  constexpr int MAX_REGS = BRINGERS > 0 ? 1 : (PIECES + 255) / 256;
+  const int stagers = (int)blockDim.x;  // threads that stage x
+  const int sid = tid;
   // One set of registers per chunk of a pass: a set that is loaded at two places of the loop gets copied by the
   // compiler right after the second load, and the copy waits for every read asked for before it, the ring's too.
   uint4 staged_sets[UNROLL][MAX_REGS];
@@ -113,7 +143,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   auto stage_load = [&](int c, uint4 (&staged)[MAX_REGS]) {
 #pragma unroll
     for (int n = 0; n < MAX_REGS; ++n) {
-      int p = tid + n * (int)blockDim.x;
+      int p = sid + n * stagers;
       p = p < PIECES ? p : PIECES - 1;
       int m = p / (SK_KC / 8);
       int k = kbeg + c * SK_KC + (p % (SK_KC / 8)) * 8;
@@ -125,7 +155,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   auto stage_store = [&](int c, int buf, uint4 (&staged)[MAX_REGS]) {
 #pragma unroll
     for (int n = 0; n < MAX_REGS; ++n) {
-      int p = tid + n * (int)blockDim.x;
+      int p = sid + n * stagers;
       p = p < PIECES ? p : PIECES - 1;  // threads past the end repeat the last piece: the same bytes to the same place
       const int m = p / (SK_KC / 8);
       const int col = (p % (SK_KC / 8)) * 8;
@@ -166,32 +196,79 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
       }
     }
   };
+  if constexpr (BRINGERS > 0) {
+    if (brings_x) {
+      // A buffer is rows of SK_ROW / 8 pieces of 16 bytes, the last of them padding; a copy fills 64 pieces in a
+      // row, wherever rows begin and end, and each lane reads the piece of x that belongs where its 16 bytes
+      // land: row min(m, M - 1), or zeros for the padding, for columns past the slice's end and behind the last row.
+      constexpr int ROW_PIECES = SK_ROW / 8;
+      constexpr int COPIES = (MT * 16 * ROW_PIECES + 63) / 64;        // copy instructions a chunk
+      constexpr int MY_COPIES = (COPIES + BRINGERS - 1) / BRINGERS;  // of one bringing wave
+      const int me = wave - waves;
+      auto bring = [&](int c, int buf) {
+#pragma unroll
+        for (int n = 0; n < MY_COPIES; ++n) {
+          int i = me + n * BRINGERS;
+          i = i < COPIES ? i : COPIES - 1;  // the last one once more: the same bytes to the same place
+          const int q = i * 64 + lane;
+          const int m = q / ROW_PIECES;
+          const int cp = q - m * ROW_PIECES;
+          const int k = kbeg + c * SK_KC + cp * 8;
+          const bool there = cp < SK_KC / 8 && k < kend && m < MT * 16;
+          const int mm = m < M ? m : M - 1;
+          const uint16_t* src = x + (size_t)mm * ldx + (k < last_k ? k : last_k);
+          sk_copy16_to_lds(there ? (const void*)src : (const void*)&sk_zeros16, &xs[buf][0][0] + i * 512);
+        }
+      };
+      // As many barriers as the waves that multiply: one after the first chunk, one after every chunk of the loop
+      // (which takes its chunks UNROLL at a time, a chunk past the slice's end included).  While chunk cc is
+      // multiplied, chunk cc + 1 arrives and chunk cc + 2 is asked for.
+      bring(0, 0);
+      bring(1, 1);
+      sk_wait_copies<MY_COPIES>();  // chunk 0 is there
+      __syncthreads();
+      const int rounds = (chunks + UNROLL - 1) / UNROLL * UNROLL;
+      int into = 2;
+      for (int cc = 0; cc < rounds; ++cc) {
+        bring(cc + 2, into);  // that buffer was last read in chunk cc - 1
+        into = into == 2 ? 0 : into + 1;
+        sk_wait_copies<MY_COPIES>();  // chunk cc + 1 is there
+        __syncthreads();
+      }
+      sk_wait_copies<0>();  // nothing lands in LDS after the block has given it back
+      return;
+    }
+  }
   // The first chunk of x and the whole ring are requested together.  The order
   // (x, then the ring's places in turn) is the one every pass of the loop below
   // leaves behind, so the compiler's count of reads in flight is exact there.
-  stage_load(0, staged_sets[0]);
+  if constexpr (BRINGERS == 0) stage_load(0, staged_sets[0]);
   asm volatile("" ::: "memory");
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
     load_w(d * 128, ring[d]);
     asm volatile("" ::: "memory");
   }
-  stage_store(0, 0, staged_sets[0]);
+  if constexpr (BRINGERS == 0) stage_store(0, 0, staged_sets[0]);
   __syncthreads();
 
+  int turn = 0;  // with three buffers: the one the next chunk lies in
   int c = 0;
   do {  // a slice has at least one chunk; a loop that may run zero times lets the first reads sink below the barrier
     // the x of the chunks after this pass's: asked for here, all of it, before the ring's reads, so that waiting
     // for it leaves those in flight; in flight while this pass's chunks are multiplied
+    if constexpr (BRINGERS == 0) {
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) stage_load(c + u + 1, staged_sets[u]);
+      for (int u = 0; u < UNROLL; ++u) stage_load(c + u + 1, staged_sets[u]);
+    }
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       // chunk c + u: its x lies in buffer `buf`, its W in the ring's places u * CH .. u * CH + CH - 1.  A chunk
       // past the slice's end (an odd number of chunks, two a pass) meets zeros of x.
       const int cc = c + u;
-      const int buf = UNROLL == 1 ? (c & 1) : (u & 1);
+      const int buf = BUFS == 3 ? turn : (UNROLL == 1 ? (c & 1) : (u & 1));
+      turn = turn == 2 ? 0 : turn + 1;
 #pragma unroll
       for (int st = 0; st < CH; ++st) {
         const int d = u * CH + st;
@@ -219,7 +296,8 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
         load_w((cc + UNROLL) * SK_KC + st * 128, ring[d]);  // the same place of the ring, a ring's length on
         asm volatile("" ::: "memory");                     // here, and not gathered at the chunk's end
       }
-      stage_store(cc + 1, buf ^ 1, staged_sets[u]);  // that buffer was last read in chunk cc - 1, before the barrier below
+      // that buffer was last read in chunk cc - 1, before the barrier below
+      if constexpr (BRINGERS == 0) stage_store(cc + 1, buf ^ 1, staged_sets[u]);
       __syncthreads();
     }
     c += UNROLL;
@@ -343,13 +421,14 @@ static int sk_launch(hipStream_t stream, const uint16_t* x, const uint16_t* w, T
   int waves, slices, len;
   rv_gemm_skinny_plan(N, K, &waves, &slices, &len);
   if (slices > 1 && part == nullptr) return rv_fail("gemm_skinny: this shape needs a workspace");
+  // a block holds SK_MAX_WAVES waves at most (two per SIMD, for their registers), the one that brings x in included
+  if (waves + SK_BRINGERS_OF(MT) > SK_MAX_WAVES) waves = SK_MAX_WAVES - SK_BRINGERS_OF(MT);
   dim3 grid(rv_div_up(rv_div_up(N, 16), waves), slices);
+  const dim3 block((waves + SK_BRINGERS_OF(MT)) * 64);  // the waves that own rows of W, and those that only bring x in
   if (tiled)
-    gemm_skinny_kernel<MT, TC, ACT, true><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc,
-                                                                               len);
+    gemm_skinny_kernel<MT, TC, ACT, true><<<grid, block, 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc, len);
   else
-    gemm_skinny_kernel<MT, TC, ACT, false><<<grid, dim3(waves * 64), 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw,
-                                                                                ldc, len);
+    gemm_skinny_kernel<MT, TC, ACT, false><<<grid, block, 0, stream>>>(x, w, out, part, M, N, K, ldx, ldw, ldc, len);
   RV_LAUNCH_CHECK("gemm_skinny");
   if (slices > 1 && do_reduce) {
     const long long total = (long long)M * N;
