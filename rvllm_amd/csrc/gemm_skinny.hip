@@ -15,7 +15,8 @@
 //   * the waves of a block own neighbouring rows and the same range of K, so
 //     they share x: the block stages x through LDS in pieces of 512 columns
 //     (double-buffered, rows padded against bank conflicts; beyond 32 rows of
-//     x in pieces of 256, brought in by waves of their own into three buffers)
+//     x in pieces of 256; beyond 16 rows brought in by waves of their own into
+//     three buffers)
 //     and every wave reads its B operands from there; up to four column sets
 //     of 16 rows of x share each read of W;
 //   * a matrix with few rows is also split along K over blocks (grid.y) so
@@ -90,14 +91,14 @@ __device__ __forceinline__ void sk_wait_copies() {
 }
 __device__ const uint4 sk_zeros16 = {0u, 0u, 0u, 0u};  // what a copy reads where x has nothing
 
-// Beyond 32 rows of x a block has three waves more, which own no rows of W and only bring x in (SK_BRINGERS_OF):
-// x is then as many bytes as W, and a wave that asks for both waits for its x behind the W it asked for earlier
+// Beyond 16 rows of x a block has three waves more, which own no rows of W and only bring x in (SK_BRINGERS_OF):
+// x is then half as many bytes as W or as many, and a wave that asks for both waits for its x behind the W it asked for earlier
 // (reads come back in the order of asking) and, with the barrier that follows, for the W of the whole next chunk
 // and of every wave of the block, which takes off the ring's depth; staging x also takes a quarter of such a
 // product's time in loads, masks and stores.  The waves that bring x in ask for nothing else, copy straight from
 // memory into LDS, a chunk ahead, and count their copies themselves; the others wait for W alone.  One such wave
 // cannot keep up with four that multiply, two nearly; with four the widest products have too few blocks.
-#define SK_BRINGERS_OF(MT) ((MT) >= 3 ? 3 : 0)
+#define SK_BRINGERS_OF(MT) ((MT) >= 2 ? 3 : 0)
 template <int MT, typename TC, int ACT = -1, bool TILED = false>
 __global__ void __launch_bounds__(SK_MAX_WAVES * 64)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, TC* __restrict__ out,
