@@ -445,6 +445,22 @@ def test_qk_norm_rope_of_a_prompt_portion(nq, nkv, hd, rot, page_size):
         assert torch.allclose(kp[page, pos % page_size].cpu().float(), k[t].float(), **tol(dtype)), t
 
 
+def test_rows_and_columns_of_a_host_matrix_copied_to_the_device():
+    """A step sends of its block tables only the requests' rows by the pages of the longest: one strided copy from
+    pinned memory, which leaves the rest of the device matrix as it was."""
+    host = torch.arange(6 * 40, dtype=torch.int32).view(6, 40).pin_memory()
+    on_device = torch.full((8, 50), -7, dtype=torch.int32, device=DEV)
+    ops.copy_rows_to_device(on_device, host, 4, 33)
+    got = on_device.cpu()
+    assert torch.equal(got[:4, :33], host[:4, :33])
+    assert (got[4:] == -7).all() and (got[:, 33:] == -7).all()
+    ops.copy_rows_to_device(on_device, host, 0, 10)  # nothing to copy is no error
+    with pytest.raises(ops.KernelError, match="pinned"):
+        ops.copy_rows_to_device(on_device, torch.zeros(6, 40, dtype=torch.int32), 2, 2)
+    with pytest.raises(ops.KernelError, match="does not fit"):
+        ops.copy_rows_to_device(on_device, host, 7, 10)
+
+
 def test_rope_table_against_64_bit_angles():
     """cos and sin of float32(position) * inv_freq, positions up to a long context, against 64-bit
     functions of the same 32-bit angle."""
