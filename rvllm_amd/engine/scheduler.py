@@ -250,6 +250,12 @@ class Scheduler:
             if not p.wants_token:
                 continue
             token = int(next_tokens[req.id])
+            if token < 0:
+                # the device found no token (a row of logits that are not numbers): the request ends here, with
+                # what it has, rather than with an id that is none in its output
+                self._finish(req, "error")
+                finished.append(req)
+                continue
             req.output.append(token)
             if not req.ignore_eos and token in req.eos_ids:
                 self._finish(req, "stop")

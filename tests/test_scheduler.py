@@ -136,6 +136,30 @@ def test_eos_stops_and_ignore_eos_does_not():
     assert done["b"].output == full and done["b"].finish_reason == "length"
 
 
+def test_a_step_that_finds_no_token_ends_its_request_with_an_error():
+    """The device's choice is -1 where a row of logits holds no number: the request ends with what it has and
+    gives its pages back; the others go on."""
+    prompt = [5, 6, 7]
+    sched, runner = build()
+    sched.add(Request("a", prompt, max_new_tokens=6))
+    sched.add(Request("b", prompt, max_new_tokens=6))
+    done = {}
+    steps = 0
+    while sched.has_work():
+        plan = sched.schedule()
+        if plan.portions:
+            chosen = runner.step(plan)
+            steps += 1
+            if steps == 3 and "a" in chosen:
+                chosen["a"] = -1
+            for r in sched.commit(plan, chosen):
+                done[r.id] = r
+    assert done["a"].finish_reason == "error" and done["a"].output == expected_output(prompt, 6)[:len(done["a"].output)]
+    assert 0 < len(done["a"].output) < 6 and all(t >= 0 for t in done["a"].output)
+    assert done["b"].output == expected_output(prompt, 6) and done["b"].finish_reason == "length"
+    assert not sched.cache.has_request("a")
+
+
 def test_context_limit_bounds_new_tokens():
     sched, runner = build(max_model_len=12)
     sched.add(Request("a", list(range(1, 10)), max_new_tokens=50))
