@@ -307,6 +307,115 @@ extern "C" int rv_topk_select(hipStream_t stream, const float* logits, int rows,
 }
 
 // ---------------------------------------------------------------------------
+// The draw on the device, from the candidates that topk_select left: what the host does with them
+// (v3/crates/rvllm-sampling/src/sampler.rs:71-135), step for step and in its order of additions, so that a
+// request gets the same tokens either way: sort by (value descending, id ascending), keep top_k, weigh by
+// exp(v - max) in 64-bit, add up from the left, cut the nucleus at the first prefix that reaches top_p of the
+// total, draw one number from the request's SplitMix64 stream and walk along the weights.  One block a row: all
+// threads sort and weigh, one thread adds and walks (the sums are one after the other by definition).  A row
+// with a candidate that is no number gets -1 and keeps its stream.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float topk_value_of(unsigned long long key) {
+  unsigned int b = (unsigned int)(key >> 32);
+  b = (b & 0x80000000u) ? (b & 0x7FFFFFFFu) : ~b;  // topk_key's order of the floats, undone
+  return __uint_as_float(b);
+}
+
+__global__ void __launch_bounds__(256)
+draw_kernel(const float* __restrict__ vals, const int* __restrict__ ids, int k, const int* __restrict__ top_k,
+            const double* __restrict__ top_p, unsigned long long* __restrict__ rng_state, int* __restrict__ chosen) {
+  __shared__ unsigned long long keys[TOPK_MAX_K];
+  __shared__ double weight[TOPK_MAX_K];
+  __shared__ int bad;
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x;
+  int padded = 1;
+  while (padded < k) padded <<= 1;
+  if (tid == 0) bad = 0;
+  __syncthreads();
+  for (int j = tid; j < padded; j += blockDim.x) {
+    unsigned long long key = 0ull;  // below every candidate's
+    if (j < k) {
+      const float v = vals[(size_t)row * k + j] + 0.0f;  // -0 as +0: the two compare equal on the host
+      if (!(fabsf(v) <= 3.402823466e38f)) bad = 1;
+      key = topk_key(v, ids[(size_t)row * k + j]);
+    }
+    keys[j] = key;
+  }
+  __syncthreads();
+  // bitonic sort, largest key first
+  for (int size = 2; size <= padded; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int t = tid; t < (padded >> 1); t += blockDim.x) {
+        const int i = 2 * t - (t & (stride - 1));
+        const int j = i + stride;
+        const unsigned long long a = keys[i], b = keys[j];
+        const bool falling = (i & size) == 0;
+        if ((a < b) == falling) {
+          keys[i] = b;
+          keys[j] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  const int n = top_k[row] > 0 ? (top_k[row] < k ? top_k[row] : k) : k;
+  const double top = (double)topk_value_of(keys[0]);
+  for (int j = tid; j < n; j += blockDim.x) weight[j] = exp((double)topk_value_of(keys[j]) - top);
+  __syncthreads();
+  if (tid != 0) return;
+  if (bad) {
+    chosen[row] = -1;
+    return;
+  }
+  double total = 0.0;
+  for (int i = 0; i < n; ++i) total += weight[i];
+  int cut = n;
+  const double p = top_p[row];
+  if (p < 1.0) {
+    const double target = (p > 0.0 ? p : 0.0) * total;
+    double cum = 0.0;
+    for (int i = 0; i < n; ++i) {
+      cum += weight[i];
+      if (cum >= target) {
+        cut = i + 1;
+        break;
+      }
+    }
+  }
+  double z = 0.0;
+  for (int i = 0; i < cut; ++i) z += weight[i];
+  unsigned long long state = rng_state[row] + 0x9E3779B97F4A7C15ull;  // SplitMix64, sampler.rs:17-36
+  rng_state[row] = state;
+  unsigned long long r = state;
+  r = (r ^ (r >> 30)) * 0xBF58476D1CE4E5B9ull;
+  r = (r ^ (r >> 27)) * 0x94D049BB133111EBull;
+  r ^= r >> 31;
+  double u = ((double)(r >> 11) * (1.0 / 9007199254740992.0)) * z;
+  int pick = cut - 1;
+  for (int i = 0; i < cut; ++i) {
+    u -= weight[i];
+    if (u <= 0.0) {
+      pick = i;
+      break;
+    }
+  }
+  chosen[row] = (int)(0xFFFFFFFFu - (unsigned int)(keys[pick] & 0xFFFFFFFFull));
+}
+
+// vals, ids [rows, k]: the candidates of topk_select (values times 1/T, any order); top_k [rows] (0: all k),
+// top_p [rows] (64-bit), rng_state [rows] (each request's stream, moved one draw on), chosen [rows].
+extern "C" int rv_draw(hipStream_t stream, const float* vals, const int* ids, int rows, int k, const int* top_k,
+                       const double* top_p, unsigned long long* rng_state, int* chosen) {
+  RV_CHECK(rows >= 0 && k >= 1 && k <= TOPK_MAX_K, "draw: k=%d must be in 1..%d (rows=%d)", k, TOPK_MAX_K, rows);
+  RV_CHECK(vals && ids && top_k && top_p && rng_state && chosen, "draw: null argument");
+  if (rows == 0) return 0;
+  draw_kernel<<<dim3(rows), dim3(256), 0, stream>>>(vals, ids, k, top_k, top_p, rng_state, chosen);
+  RV_LAUNCH_CHECK("draw");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // From one decode step to the next without the host: every request's chosen
 // token becomes its next token, one position on.  A step of decoded tokens is
 // described by these arrays alone (token t belongs to request t), so the same

@@ -23,7 +23,7 @@ import torch
 
 from ..config.engine_config import EngineConfig
 from ..sampling.params import SamplingParams
-from ..sampling.sampler import Sampler
+from ..sampling.sampler import DeviceDraws, Sampler
 from .runner import ModelRunner
 from .scheduler import PlannedPortion, Request, RequestState, Scheduler, StepPlan
 
@@ -91,7 +91,7 @@ class LLMEngine:
             if p.wants_token:
                 wanting.append(p.request)
         self.plans += 1
-        ahead = self._greedy_steps_ahead(plan)
+        ahead = self._steps_ahead(plan)
         if ahead > 1:
             return results + self._decode_ahead(plan, ahead)
         try:
@@ -110,16 +110,20 @@ class LLMEngine:
         finished = self.scheduler.commit(plan, next_tokens)
         return results + [self._result(r) for r in finished]
 
-    # ---- several greedy steps from one plan ------------------------------
-    def _greedy_steps_ahead(self, plan: StepPlan) -> int:
+    # ---- several decode steps from one plan ------------------------------
+    def _steps_ahead(self, plan: StepPlan) -> int:
         """How many decode steps may follow one another from this plan: more
-        than one only if every request in it decodes greedily, none could end
-        by its length or the model's on the way, nothing was set back, and no
-        request waits for which there is a place (it would be admitted that
-        much later; with every place taken, the most a waiting request can
-        lose is the few steps by which an end id is noticed late).  A request
-        that meets an end id on the way stops there; what was run for it after
-        that is dropped, and costs the others nothing."""
+        than one only if every request in it decodes one token and gets its
+        next one chosen on the device (the arg-max, or a draw as the host
+        draws, for which the requests that sample must ask for the same number
+        of candidates), none could end by its length or the model's on the
+        way, nothing was set back, and no request waits for which there is a
+        place (it would be admitted that much later; with every place taken,
+        the most a waiting request can lose is the few steps by which an end
+        id is noticed late).  A request that meets an end id on the way stops
+        there; what was run for it after that is dropped, its stream of
+        numbers stands after its last token's draw, and it costs the others
+        nothing."""
         ahead = self.runner.config.greedy_steps_ahead
         if ahead <= 1 or plan.set_back:
             return 1
@@ -127,13 +131,23 @@ class LLMEngine:
             return 1
         for p in plan.portions:
             req = p.request
-            if p.count != 1 or not p.wants_token or not req.params.is_greedy():
+            if p.count != 1 or not p.wants_token:
                 return 1
             ahead = min(ahead, req.max_new_tokens - len(req.output), self.scheduler.max_model_len - req.total)
+        # requests that sample are drawn for on the device, if they ask for the same number of candidates
+        params = [p.request.params for p in plan.portions]
+        if not all(sp.is_greedy() for sp in params) and not DeviceDraws.usable(self.sampler.vocab_size, params):
+            return 1
         return max(1, ahead)
 
     def _decode_ahead(self, plan: StepPlan, ahead: int) -> list[GenerationResult]:
-        rows = self.runner.decode_greedy([(p.request.id, p.request.tokens_at(p.start, 1)[0]) for p in plan.portions], ahead)
+        requests = [p.request for p in plan.portions]
+        choose = None
+        if not all(r.params.is_greedy() for r in requests):
+            choose = DeviceDraws(self.sampler.vocab_size, [r.params for r in requests], [r.rng for r in requests],
+                                 self.runner.device)
+        rows = self.runner.decode_ahead([(p.request.id, p.request.tokens_at(p.start, 1)[0]) for p in plan.portions],
+                                        ahead, choose)
         finished: list[Request] = []
         for i, row in enumerate(rows):
             live = [(p, token) for p, token in zip(plan.portions, row) if p.request.state is RequestState.RUNNING]
@@ -142,6 +156,9 @@ class LLMEngine:
             self.steps += 1
             self.tokens_run += len(live)
             step_plan = StepPlan([PlannedPortion(p.request, p.start + i, 1, True) for p, _ in live], [], [])
+            for p, token in live:
+                if token >= 0 and not p.request.params.is_greedy():
+                    p.request.rng.next_u64()  # the draw that the device made for this token
             finished += self.scheduler.commit(step_plan, {p.request.id: token for p, token in live})
         return [self._result(r) for r in finished]
 

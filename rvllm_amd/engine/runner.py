@@ -291,12 +291,18 @@ class ModelRunner:
 
     # ---- several greedy decode steps without the host in between ---------
     def decode_greedy(self, entries: Sequence[tuple[Hashable, int]], steps: int) -> list[list[int]]:
+        """``decode_ahead`` with the arg-max as the choice."""
+        return self.decode_ahead(entries, steps)
+
+    def decode_ahead(self, entries: Sequence[tuple[Hashable, int]], steps: int, choose=None) -> list[list[int]]:
         """``entries``: (request, its next token), one decoded token each.
         Runs up to ``steps`` decode steps one after the other, each request's
-        arg-max token becoming its next token on the device, and returns the
+        chosen token becoming its next token on the device, and returns the
         chosen tokens step by step, ``[steps run][request]``: the same tokens
-        as as many calls of ``step`` with an arg-max each, with one wait for
-        the device instead of one a step.
+        as as many calls of ``step`` with a choice each, with one wait for
+        the device instead of one a step.  ``choose(logits, out)`` writes a
+        token id for every row of the 32-bit logits into ``out`` on the device
+        (``sampling.sampler.DeviceDraws``); without it, the arg-max.
 
         The steps after the first replay the graph captured for the shape, so
         fewer than ``steps`` are run (at least one) where there is none yet,
@@ -323,7 +329,10 @@ class ModelRunner:
             if i > 0:
                 ops.advance_decode(batch, chosen[i - 1])
             logits = self._forward(batch) if i == 0 else self._replay(key)
-            ops.argmax(logits, out=chosen[i])
+            if choose is None:
+                ops.argmax(logits, out=chosen[i])
+            else:
+                choose(logits, chosen[i])
         for p in portions:
             self.cache.commit(p.request, p.start + run)
         return chosen.cpu().tolist()

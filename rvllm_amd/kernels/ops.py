@@ -652,6 +652,27 @@ def topk_select(logits: torch.Tensor, k: int, inv_temp: torch.Tensor) -> tuple[t
     return vals, idx
 
 
+def draw(vals: torch.Tensor, ids: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, rng_state: torch.Tensor,
+         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token a row from the candidates ``vals, ids [rows, k]`` of ``topk_select``, drawn on the device as the
+    host draws (``sampling.sampler.sample_rows``): ``top_k`` int32 and ``top_p`` float64 a row, ``rng_state`` int64
+    a row, each request's SplitMix64 state, which moves one draw on.  -1 for a row whose candidates are not all
+    numbers."""
+    _gpu(vals, ids, top_k, top_p, rng_state, out)
+    rows, k = vals.shape
+    _need(vals.dtype == torch.float32 and ids.dtype == torch.int32 and ids.shape == vals.shape,
+          "draw: float32 values and int32 ids [rows, k] expected")
+    _need(top_k.dtype == torch.int32 and top_p.dtype == torch.float64 and rng_state.dtype == torch.int64
+          and top_k.numel() == rows and top_p.numel() == rows and rng_state.numel() == rows,
+          "draw: top_k int32, top_p float64 and rng_state int64, one a row, expected")
+    if out is None:
+        out = torch.empty(rows, dtype=torch.int32, device=vals.device)
+    _need(out.dtype == torch.int32 and out.numel() == rows, "draw: int32 out, one a row, expected")
+    _check(library().rv_draw(_stream(), _ptr(vals), _ptr(ids), _c_int(rows), _c_int(k), _ptr(top_k), _ptr(top_p),
+                             _ptr(rng_state), _ptr(out)))
+    return out
+
+
 def gemm_bf16(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,
               out_dtype: Optional[torch.dtype] = None, sliced_ok: bool = False):
     """out = x @ w^T on the matrix cores for bf16 inputs; None when no

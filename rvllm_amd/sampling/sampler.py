@@ -126,6 +126,41 @@ def sample_rows(vals: np.ndarray, ids: np.ndarray, top_k: Sequence[int], top_p: 
     return pool[np.arange(rows), chosen].tolist()
 
 
+class DeviceDraws:
+    """The next tokens of a fixed set of requests, chosen on the device step after step without the host:
+    ``topk_select`` and then ``ops.draw``, which does what ``sample_rows`` does with each request's stream of
+    numbers kept on the device.  Rows that decode greedily are rows that keep one candidate.  Possible while the
+    rows that sample ask for the same number of candidates (``usable``); a row whose largest logits are not all
+    numbers gets -1 (the arg-max skips such logits, the host's draw refuses them)."""
+
+    def __init__(self, vocab_size: int, params: Sequence[SamplingParams], rngs: Sequence[SplitMix64], device):
+        ks = {p.kernel_k(vocab_size) for p in params if not p.is_greedy()}
+        if len(ks) != 1:
+            raise SamplingError("the rows that sample must ask for the same number of candidates")
+        self.k = ks.pop()
+        greedy = [p.is_greedy() for p in params]
+        self.inv_temp = torch.tensor([1.0 if g else 1.0 / p.temperature for p, g in zip(params, greedy)],
+                                     dtype=torch.float32, device=device)
+        self.top_k = torch.tensor([1 if g else p.top_k for p, g in zip(params, greedy)], dtype=torch.int32,
+                                  device=device)
+        self.top_p = torch.tensor([1.0 if g else p.top_p for p, g in zip(params, greedy)], dtype=torch.float64,
+                                  device=device)
+        # the streams' states as signed 64-bit numbers, which is what the tensor holds
+        self.state = torch.tensor([r.state - (1 << 64) if r.state >= (1 << 63) else r.state for r in rngs],
+                                  dtype=torch.int64, device=device)
+
+    @staticmethod
+    def usable(vocab_size: int, params: Sequence[SamplingParams]) -> bool:
+        try:
+            return len({p.kernel_k(vocab_size) for p in params if not p.is_greedy()}) == 1
+        except SamplingError:
+            return False
+
+    def __call__(self, logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        vals, ids = ops.topk_select(logits, self.k, self.inv_temp)
+        return ops.draw(vals, ids, self.top_k, self.top_p, self.state, out)
+
+
 class Sampler:
     """Next tokens for the rows of a step's logits."""
 

@@ -823,6 +823,42 @@ def test_topk_select(vocab, k):
         assert torch.equal(vals[r], x[r][idx[r]] * inv_t[r])
 
 
+@pytest.mark.parametrize("k", [1, 7, 50, 509, 1024])
+def test_the_draw_on_the_device_is_the_hosts(k):
+    """The device sorts, weighs, cuts and walks as the host does, with the same stream of numbers: the same tokens
+    row by row and draw after draw.  Rows with every kind of cut (all candidates, the first only, a few, a nucleus
+    from 0 to 1), equal values among the candidates (the lower id first), values far apart (weights that vanish)
+    and both zeros."""
+    from rvllm_amd.sampling.sampler import SplitMix64, sample_rows
+
+    rows = 24
+    g = torch.Generator().manual_seed(50 + k)
+    vals = torch.randn(rows, k, generator=g) * 3
+    vals[1] = (vals[1] * 2).round() / 2  # many equal values
+    vals[2] = vals[2] * 40  # exp underflows for most
+    if k > 2:
+        vals[3, :2] = torch.tensor([0.0, -0.0])
+    ids = torch.stack([torch.randperm(70000, generator=g)[:k] for _ in range(rows)]).int()
+    top_k = [[0, 1, min(k, 5), k][r % 4] for r in range(rows)]
+    top_p = [[1.0, 0.9, 0.5, 0.0, 0.999999, 0.3][r % 6] for r in range(rows)]
+    seeds = [(0x9E3779B97F4A7C15 * (r + 1)) & ((1 << 64) - 1) for r in range(rows)]
+    rngs = [SplitMix64(s) for s in seeds]
+    state = dev(torch.tensor([s - (1 << 64) if s >= (1 << 63) else s for s in seeds], dtype=torch.int64))
+    d_vals, d_ids = dev(vals), dev(ids)
+    d_k, d_p = dev(torch.tensor(top_k, dtype=torch.int32)), dev(torch.tensor(top_p, dtype=torch.float64))
+    for draw in range(6):
+        want = sample_rows(vals.numpy(), ids.numpy(), top_k, top_p, rngs, 70000)
+        got = ops.draw(d_vals, d_ids, d_k, d_p, state).cpu().tolist()
+        assert got == want, f"draw {draw}"
+    # the streams stand where the host's stand
+    assert [s & ((1 << 64) - 1) for s in state.cpu().tolist()] == [r.state for r in rngs]
+    # a candidate that is no number: no token, and the stream stays
+    vals[0, 0] = float("nan")
+    before = state.clone()
+    got = ops.draw(dev(vals), d_ids, d_k, d_p, state).cpu().tolist()
+    assert got[0] == -1 and all(t >= 0 for t in got[1:]) and state[0] == before[0] and (state[1:] != before[1:]).all()
+
+
 def test_kernels_refuse_what_they_cannot_do():
     x = torch.randn(4, 32)
     with pytest.raises(ops.KernelError, match="GPU"):
