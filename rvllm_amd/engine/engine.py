@@ -115,8 +115,7 @@ class LLMEngine:
         """How many decode steps may follow one another from this plan: more
         than one only if every request in it decodes one token and gets its
         next one chosen on the device (the arg-max, or a draw as the host
-        draws, for which the requests that sample must ask for the same number
-        of candidates), none could end by its length or the model's on the
+        draws), none could end by its length or the model's on the
         way, nothing was set back, and no request waits for which there is a
         place (it would be admitted that much later; with every place taken,
         the most a waiting request can lose is the few steps by which an end
@@ -134,7 +133,7 @@ class LLMEngine:
             if p.count != 1 or not p.wants_token:
                 return 1
             ahead = min(ahead, req.max_new_tokens - len(req.output), self.scheduler.max_model_len - req.total)
-        # requests that sample are drawn for on the device, if they ask for the same number of candidates
+        # requests that sample are drawn for on the device (not with parameters that the host's draw refuses too)
         params = [p.request.params for p in plan.portions]
         if not all(sp.is_greedy() for sp in params) and not DeviceDraws.usable(self.sampler.vocab_size, params):
             return 1

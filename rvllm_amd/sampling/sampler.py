@@ -129,15 +129,16 @@ def sample_rows(vals: np.ndarray, ids: np.ndarray, top_k: Sequence[int], top_p: 
 class DeviceDraws:
     """The next tokens of a fixed set of requests, chosen on the device step after step without the host:
     ``topk_select`` and then ``ops.draw``, which does what ``sample_rows`` does with each request's stream of
-    numbers kept on the device.  Rows that decode greedily are rows that keep one candidate.  Possible while the
-    rows that sample ask for the same number of candidates (``usable``); a row whose largest logits are not all
-    numbers gets -1 (the arg-max skips such logits, the host's draw refuses them)."""
+    numbers kept on the device.  The device selects as many candidates for every row as the row that asks for
+    most; a row keeps its own ``top_k`` of them after the sort, which are the ones it would have had selected
+    (equal values go by the lower id both times), and rows that decode greedily keep one.  A row whose largest
+    logits are not all numbers gets -1 (the arg-max skips such logits, the host's draw refuses them)."""
 
     def __init__(self, vocab_size: int, params: Sequence[SamplingParams], rngs: Sequence[SplitMix64], device):
-        ks = {p.kernel_k(vocab_size) for p in params if not p.is_greedy()}
-        if len(ks) != 1:
-            raise SamplingError("the rows that sample must ask for the same number of candidates")
-        self.k = ks.pop()
+        ks = [p.kernel_k(vocab_size) for p in params if not p.is_greedy()]
+        if not ks:
+            raise SamplingError("no row samples")
+        self.k = max(ks)
         greedy = [p.is_greedy() for p in params]
         self.inv_temp = torch.tensor([1.0 if g else 1.0 / p.temperature for p, g in zip(params, greedy)],
                                      dtype=torch.float32, device=device)
@@ -151,8 +152,9 @@ class DeviceDraws:
 
     @staticmethod
     def usable(vocab_size: int, params: Sequence[SamplingParams]) -> bool:
+        """Whether some row samples and every such row's parameters are ones the device selects for."""
         try:
-            return len({p.kernel_k(vocab_size) for p in params if not p.is_greedy()}) == 1
+            return len([p.kernel_k(vocab_size) for p in params if not p.is_greedy()]) > 0
         except SamplingError:
             return False
 

@@ -259,9 +259,8 @@ def test_greedy_steps_ahead_change_no_token(model_dirs, name):
     that end at different lengths, one of them at an end id met on the way, and with so few pages that requests are
     set back.  With requests that sample among them the steps still follow one another: the device then draws for
     them as the host does, from each request's own stream of numbers, so the tokens are those of single steps with
-    the host's draw (temperatures, nucleus and seeds that differ); only requests that ask for different numbers of
-    candidates have every step planned by itself.  (The engine against the engine: what a single step computes is
-    held to the plain model by the replay tests.)"""
+    the host's draw (temperatures, nucleus, seeds and numbers of candidates that differ).  (The engine against the
+    engine: what a single step computes is held to the plain model by the replay tests.)"""
     def run(ahead, tight, places=4):
         engine = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(
             dtype="bfloat16", max_model_len=200, max_num_seqs=places, max_num_batched_tokens=64, max_prefill_chunk=64,
@@ -296,13 +295,10 @@ def test_greedy_steps_ahead_change_no_token(model_dirs, name):
     assert [single[("all greedy", j)][1] for j in (0, 2, 3)] == ["length"] * 3
     assert e4.steps == e1.steps  # a step is a step, however many were planned at once
     assert e1.plans == e1.steps and e4.plans < 0.7 * e4.steps
-    for phase in ("one samples", "three sample"):  # steps follow one another with draws on the device
+    for phase in ("one samples", "three sample", "other candidates"):  # steps follow one another with draws on the device
         plans, steps = run.planned[(4, False, 4, phase)]
         assert plans < 0.7 * steps, phase
         assert single[(phase, 2)][0] != single[("all greedy", 2)][0]  # and the draws are draws
-    plans, steps = run.planned[(4, False, 4, "other candidates")]
-    # while both requests that sample run (the 23 tokens of the shorter one), every step is planned by itself
-    assert plans >= 23 and plans > run.planned[(4, False, 4, "three sample")][0]
     # Where requests are set back or wait for a place, steps that follow one another notice an end a few steps
     # late, so the requests share their steps differently; the logits then differ in their last bits (the
     # attention's split of the keys and the products' kernels go by what a step holds), which the arg-max does

@@ -150,13 +150,13 @@ def test_rows_drawn_together_refuse_what_one_row_refuses():
 
 
 def test_when_the_device_can_draw_for_a_step():
-    """Steps follow one another for requests that sample while these ask the device for the same number of
-    candidates; greedy requests among them do not count (they keep one candidate of however many)."""
+    """Steps follow one another for requests that sample, whatever numbers of candidates they ask for (the device
+    selects as many as the one that asks for most; each keeps its own); greedy requests among them keep one."""
     from rvllm_amd.sampling.sampler import DeviceDraws
 
     greedy, a, b = SamplingParams(), SamplingParams(0.8, 20, 0.9, seed=1), SamplingParams(1.2, 20, 1.0, seed=2)
     assert DeviceDraws.usable(1000, [a, b, greedy])
-    assert not DeviceDraws.usable(1000, [a, SamplingParams(0.8, 50, 1.0)])
+    assert DeviceDraws.usable(1000, [a, SamplingParams(0.8, 50, 1.0)])
     assert not DeviceDraws.usable(1000, [greedy, greedy])  # nothing to draw: the arg-max does it
     assert DeviceDraws.usable(300, [SamplingParams(0.8, 0, 1.0), greedy])  # the whole of a small vocabulary
     assert not DeviceDraws.usable(5000, [SamplingParams(0.8, 0, 1.0)])  # refused for a large one, as on the host
