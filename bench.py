@@ -332,6 +332,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-probes", action="store_true", help="skip the measured peaks (read rate, library product)")
+    ap.add_argument("--page-size", type=int, default=16, choices=[16, 32, 64], help="tokens a page of the cache holds")
     ap.add_argument("--sampled", action="store_true", help="the decode steps draw their tokens (temperature 0.8 among "
                     "the 50 largest logits) instead of taking the arg-max; the metric then says so")
     ap.add_argument("--graphs", type=int, default=1, help="replay decode steps from captured HIP graphs (0 = off)")
@@ -363,7 +364,7 @@ def main() -> int:
     max_batch = max(args.batch, 1 if args.no_points else 64)
     steps_total = args.steps + args.warmup + 8
     engine_cfg = EngineConfig(
-        dtype=args.dtype, page_size=16, max_model_len=max(args.context + steps_total, args.prefill_at + args.prefill_tokens),
+        dtype=args.dtype, page_size=args.page_size, max_model_len=max(args.context + steps_total, args.prefill_at + args.prefill_tokens),
         max_num_seqs=max_batch, max_num_batched_tokens=max(args.prefill_tokens, max_batch),
         max_prefill_chunk=max(args.prefill_tokens, 1), max_cache_tokens=max(max_batch * (args.context + steps_total + 16), args.prefill_at + args.prefill_tokens + 64),
         use_graphs=bool(args.graphs),
