@@ -1,5 +1,6 @@
 """A plain, slow implementation of the Gemma dense text decoder: whole
-sequences, no cache, one function per part, PyTorch on the CPU.  It shares no
+sequences, no cache, one function per part, plain PyTorch operations (on the CPU
+unless a test of many thousand tokens names another device).  It shares no
 code with the engine; the tests compare the engine against it.
 
 Every function is written from the reference's formulas and cites them
@@ -99,19 +100,27 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, w
     nkv = k.shape[1]
     group = nq // nkv
     out = torch.empty_like(q)
-    pos = torch.arange(T)
-    visible = pos[None, :] <= pos[:, None]
-    if window is not None:
-        visible &= pos[None, :] >= pos[:, None] - window + 1
-    for h in range(nq):
-        kh = h // group
-        s = scale * (q[:, h, :] @ k[:, kh, :].T)  # [T, T]
-        s = s.masked_fill(~visible, float("-inf"))
-        s = s - s.max(dim=-1, keepdim=True).values
-        p = torch.exp(s)
-        p = p / p.sum(dim=-1, keepdim=True)
-        out[:, h, :] = p @ v[:, kh, :]
+    pos = torch.arange(T, device=q.device)
+    # Rows are taken ROWS_AT_A_TIME at a time, so that a long sequence needs no T x T table; a row's result does
+    # not depend on the cut (every visible key of a row is in its piece, the others weigh exp(-inf) = 0).
+    for r0 in range(0, T, ROWS_AT_A_TIME):
+        r1 = min(T, r0 + ROWS_AT_A_TIME)
+        c0 = 0 if window is None else max(0, r0 - window + 1)
+        visible = pos[None, c0:r1] <= pos[r0:r1, None]
+        if window is not None:
+            visible &= pos[None, c0:r1] >= pos[r0:r1, None] - window + 1
+        for h in range(nq):
+            kh = h // group
+            s = scale * (q[r0:r1, h, :] @ k[c0:r1, kh, :].T)  # [rows, keys]
+            s = s.masked_fill(~visible, float("-inf"))
+            s = s - s.max(dim=-1, keepdim=True).values
+            p = torch.exp(s)
+            p = p / p.sum(dim=-1, keepdim=True)
+            out[r0:r1, h, :] = p @ v[c0:r1, kh, :]
     return out
+
+
+ROWS_AT_A_TIME = 2048
 
 
 def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
@@ -175,7 +184,7 @@ def layer(x, positions, w: dict, p: str, cfg: dict, kind: str) -> torch.Tensor:
     else:
         inv_freq = rope_inv_freq(hd, cfg["theta_global"], cfg["factor"])
         window = None
-    inv_freq = inv_freq.to(torch.float64 if x.dtype == torch.float64 else torch.float32)
+    inv_freq = inv_freq.to(device=x.device, dtype=torch.float64 if x.dtype == torch.float64 else torch.float32)
     q = rope(q, positions, inv_freq)
     k = rope(k, positions, inv_freq)
     a = attention(q, k, v, float(cfg["qpas"]) ** -0.5, window).reshape(T, nq * hd)
@@ -186,15 +195,17 @@ def layer(x, positions, w: dict, p: str, cfg: dict, kind: str) -> torch.Tensor:
     return x + rmsnorm(f, w[f"{p}.post_feedforward_layernorm.weight"], eps)
 
 
-def forward(weights: dict, cfg: dict, token_ids, dtype=torch.float32) -> torch.Tensor:
+def forward(weights: dict, cfg: dict, token_ids, dtype=torch.float32, device="cpu") -> torch.Tensor:
     """Logits [T, vocab] of a whole sequence.  Embedding times sqrt(hidden)
     (v3/crates/rvllm-loader/src/gemma4_load.rs:233-246, metal_host.rs:298); the
     layers; final norm; head against the *unscaled* embedding table when tied
-    (gemma4_load.rs:431-457); optional soft-cap."""
-    w = {k: v.to(dtype) for k, v in weights.items()}
+    (gemma4_load.rs:431-457); optional soft-cap.  ``device``: where these plain
+    tensor operations run (sequences of many thousand tokens take the CPU minutes); the
+    result comes back to the CPU."""
+    w = {k: v.to(device=device, dtype=dtype) for k, v in weights.items()}
     pre = find_prefix(w)
-    ids = torch.as_tensor(list(token_ids), dtype=torch.long)
-    positions = torch.arange(len(ids))
+    ids = torch.as_tensor(list(token_ids), dtype=torch.long, device=device)
+    positions = torch.arange(len(ids), device=device)
     emb = w[f"{pre}.embed_tokens.weight"]
     x = emb[ids] * torch.tensor(math.sqrt(cfg["hidden"]), dtype=torch.float32).to(dtype)
     for l in range(cfg["layers"]):
@@ -204,7 +215,7 @@ def forward(weights: dict, cfg: dict, token_ids, dtype=torch.float32) -> torch.T
     logits = x @ head.T
     if cfg["softcap"] is not None:
         logits = softcap(logits, cfg["softcap"])
-    return logits
+    return logits.cpu()
 
 
 def load_weights(model_dir) -> dict:

@@ -600,6 +600,33 @@ def test_paged_attention_mfma(nq, nkv, hd, window, page_size, kernels):
     assert torch.allclose(case.run("mfma", hd ** -0.5, **kw).float(), want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,hd", [(4, 2, 320), (2, 1, 512), (34, 2, 272)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_paged_attention_generic_above_256(dtype, nq, nkv, hd, window):
+    """Head sizes that no matrix-core kernel takes, up to the largest allowed, and 17 query heads a group."""
+    case = Case(MIXED, nq, nkv, hd, 16, dtype, 23, window)
+    got = case.run("generic", hd ** -0.5)
+    assert torch.allclose(got.float(), case.reference(hd ** -0.5).float(), **tol(dtype))
+    kp, vp = to_cache(case.k_log, case.v_log)
+    assert not ops.mfma_attention_covers(kp, vp, nq)
+    with pytest.raises(ops.KernelError):
+        Case([(5, 1)], 1, 1, 528, 16, dtype, 23).run("generic", 1.0)  # beyond the largest head size: refused
+
+
+@pytest.mark.parametrize("nq,nkv,hd", [(8, 4, 256), (32, 16, 128), (6, 1, 48)])
+@pytest.mark.parametrize("window", [None, 100, 1024])
+def test_paged_attention_mfma_many_single_tokens_beside_long_portions(nq, nkv, hd, window):
+    """A step as a scheduler builds it under load: twenty decoding requests at contexts from a few keys to over
+    a thousand, between and around two long prompt portions (one from position 0, one continuing): one launch
+    of each attention kernel, each leaving the other's requests alone."""
+    singles = [(3 + 61 * i, 1) for i in range(20)]
+    portions = singles[:7] + [(0, 300)] + singles[7:15] + [(517, 200)] + singles[15:]
+    case = Case(portions, nq, nkv, hd, 16, torch.bfloat16, 24, window)
+    want = case.reference(hd ** -0.5).float()
+    assert torch.allclose(case.run("mfma", hd ** -0.5).float(), want, **tol(torch.bfloat16))
+
+
 def test_paged_attention_shared_tiles_long_prompt_portions():
     """Portions as a scheduler cuts a long prompt: from position 0, continuing
     at an odd position, and one that passes a window's edge."""

@@ -147,6 +147,61 @@ def test_more_decoding_requests_than_the_few_row_product_takes(model_dirs, plain
         tt.compare(got[rid], want, dtype, f"{name} {count} requests {rid}")
 
 
+# ---- the steps a scheduler builds under load: dozens of decoders beside a long portion ------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_dozens_of_decoding_requests_beside_a_long_portion(model_dirs, plain_models, name, dtype):
+    """44 requests through the engine with a budget of 100 tokens a step and portions of at most 64: most have
+    short prompts and are soon decoding, the others' prompts of 130 to 200 tokens then arrive in portions beside
+    thirty and more decoded tokens, so that one step runs both attention kernels (and the library's products,
+    where the step has more than 64 rows).  Every token is the plain implementation's."""
+    weights, cfg = plain_models[name]
+    rng = np.random.default_rng(44)
+    lengths = [int(rng.integers(2, 12)) for _ in range(36)] + [130, 200, 177, 64, 150, 199, 131, 166]
+    prompts = list(tt.make_sequences(cfg["vocab"], lengths, seed=44).values())
+    new = 30
+    engine = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(
+        dtype=dtype, max_model_len=256, max_num_seqs=44, max_num_batched_tokens=100, max_prefill_chunk=64))
+    shapes = []
+    run_step = engine.runner.step
+
+    def watched(entries, **kw):
+        shapes.append((sum(len(tokens) == 1 for _, tokens, _ in entries), max(len(tokens) for _, tokens, _ in entries)))
+        return run_step(entries, **kw)
+
+    engine.runner.step = watched
+    results = engine.generate(prompts, None, max_new_tokens=new, ignore_eos=True)
+    assert any(singles >= 30 and longest >= 60 for singles, longest in shapes), shapes
+    assert sum(singles >= 30 and longest >= 16 for singles, longest in shapes) >= 10
+    from test_gpu_generate import assert_greedy
+
+    for prompt, res in zip(prompts, results):
+        assert len(res.tokens) == new and res.set_backs == 0
+        assert_greedy(weights, cfg, prompt, res.tokens, dtype)
+    if dtype == "float32":
+        for prompt, res in list(zip(prompts, results))[::4]:
+            assert res.tokens == plain_gemma.greedy(weights, cfg, prompt, new, torch.float64)
+
+
+# ---- heads that only the kernel for any size takes -----------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "mixed"])
+def test_a_head_size_above_256_and_17_query_heads_a_group(tmp_path, dtype, mode):
+    """Head size 272 with 34 query heads on 2 key/value heads: neither matrix-core attention kernel takes these,
+    so bf16 too runs the one for any size; the q/k norm takes its path for odd sizes."""
+    folder = tiny_models.write_model(tmp_path / "G", "G")
+    weights, cfg = plain_gemma.load_weights(folder), plain_gemma.read_config(folder)
+    seqs = tt.make_sequences(cfg["vocab"], [3, 40, 77, 130], seed=7)
+    steps = (tt.trace_whole if mode == "whole" else tt.trace_mixed)(seqs)
+    runner = runner_for(folder, dtype, tt.required_tokens(steps))
+    view = runner.storage.views[0]
+    assert not ops.mfma_attention_covers(view.k_pages, view.v_pages, cfg["nq"])
+    got = tt.collect(steps, tt.run_in_process(runner, steps), cfg["vocab"])
+    prefix = steps[0]["entries"][0]["id"].split("-")[0]
+    for rid, ids in seqs.items():
+        tt.compare(got[f"{prefix}-{rid}"], plain_gemma.forward(weights, cfg, ids, torch.float64), dtype, f"G {mode} {rid}")
+
+
 # ---- a folder in several shards ------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_folder_in_three_shards(model_dirs, plain_models, tmp_path, dtype):

@@ -155,8 +155,35 @@ CONFIG_4B = {
     "final_logit_softcapping": None,
 }
 
+# E's layers for sequences of many thousand tokens.
+CONFIG_LONG = dict(CONFIG_E, max_position_embeddings=32768)
+
+# Heads that the matrix-core attention kernels do not take, so that bf16 runs the kernel for any size too: a head
+# size above 256 (and no multiple of 32), 17 query heads on each key/value head.
+CONFIG_G = {
+    "architectures": ["Gemma3ForCausalLM"],
+    "num_hidden_layers": 2,
+    "layer_types": ["full_attention", "sliding_attention"],
+    "hidden_size": 112,
+    "num_attention_heads": 34,
+    "num_key_value_heads": 2,
+    "head_dim": 272,
+    "intermediate_size": 200,
+    "vocab_size": 333,
+    "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 1024,
+    "sliding_window": 33,
+    "rope_theta": 1000000.0,
+    "rope_local_base_freq": 10000.0,
+    "rope_scaling": {"rope_type": "linear", "factor": 2.0},
+    "query_pre_attn_scalar": 100,
+    "hidden_activation": "gelu_pytorch_tanh",
+    "tie_word_embeddings": True,
+    "final_logit_softcapping": None,
+}
+
 CONFIGS = {"A": (CONFIG_A, 0), "B": (CONFIG_B, 1), "C": (CONFIG_C, 2)}
-LARGER = {"D": (CONFIG_D, 3), "E": (CONFIG_E, 4), "4B": (CONFIG_4B, 5)}
+LARGER = {"D": (CONFIG_D, 3), "E": (CONFIG_E, 4), "4B": (CONFIG_4B, 5), "LONG": (CONFIG_LONG, 6), "G": (CONFIG_G, 7)}
 
 
 def write_model(folder, name: str, dtype=torch.bfloat16, seed=None) -> Path:
