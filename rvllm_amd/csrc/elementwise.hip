@@ -517,3 +517,38 @@ extern "C" int rv_softcap(hipStream_t stream, float* logits, long long total, fl
   RV_LAUNCH_CHECK("softcap");
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// bias of a projection, in place: x[r][c] += bias[c], the sum in 32-bit.  With `slices` > 0, x is the result of
+// adding up that many 32-bit partial sums [slices][rows][width] (the K slices of a product) and the bias.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ part, int slices, const void* __restrict__ bias,
+                                int bias_f32, long long total, int width) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float v;
+  if (slices > 0) {
+    v = 0.f;
+    for (int s = 0; s < slices; ++s) v += part[(long long)s * total + idx];
+  } else {
+    v = rv_to_float(x[idx]);
+  }
+  x[idx] = rv_from_float<T>(v + rv_load_w(bias, bias_f32, (int)(idx % width)));
+}
+
+extern "C" int rv_add_bias(hipStream_t stream, void* x, int dtype, const float* part, int slices, const void* bias,
+                           int bias_f32, int rows, int width) {
+  RV_CHECK(rows >= 0 && width > 0 && x && bias && slices >= 0 && (slices == 0 || part), "add_bias: bad arguments");
+  if (rows == 0) return 0;
+  const long long total = (long long)rows * width;
+  dim3 grid(rv_div_up(total, 256)), block(256);
+  if (dtype == RV_F32)
+    add_bias_kernel<float><<<grid, block, 0, stream>>>((float*)x, part, slices, bias, bias_f32, total, width);
+  else if (dtype == RV_BF16)
+    add_bias_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)x, part, slices, bias, bias_f32, total, width);
+  else
+    return rv_fail("add_bias: unsupported dtype %d", dtype);
+  RV_LAUNCH_CHECK("add_bias");
+  return 0;
+}

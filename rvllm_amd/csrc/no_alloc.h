@@ -20,12 +20,22 @@
 //     stream follow one another and are safe.
 //   * The device that is current when the call is made must be the device of
 //     the stream and of the pointers.
+//   * The address of the array on a device is looked up once per device, which
+//     may load the library's code onto that device: rv_no_alloc_init() does it
+//     for the current device.  A caller that will call rv_argmax_no_alloc while
+//     a stream is being captured, or from a place where nothing may be loaded,
+//     calls rv_no_alloc_init() first, once per device, outside any capture.
+//     Without it the first rv_argmax_no_alloc on a device does the same look-up
+//     itself, and must then not be made under capture.
 #pragma once
 
 #include <hip/hip_runtime.h>
 
 #define RV_NO_ALLOC_MAX_ROWS 256
 #define RV_NO_ALLOC_MAX_PARTS 256
+
+// Looks the array's address up for the current device (once; later calls return at once).  0 or an error code.
+extern "C" int rv_no_alloc_init(void);
 
 extern "C" int rv_argmax_no_alloc(hipStream_t stream, const float* logits, int rows, int vocab, long long row_stride,
                                   int* out);

@@ -147,6 +147,8 @@ static void* scratch_on_current_device() {
   return g_scratch_ptr[dev];
 }
 
+extern "C" int rv_no_alloc_init(void) { return scratch_on_current_device() ? 0 : -1; }
+
 extern "C" int rv_argmax_no_alloc(hipStream_t stream, const float* logits, int rows, int vocab, long long row_stride,
                                   int* out) {
   RV_CHECK(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax_no_alloc: bad sizes rows=%d vocab=%d", rows, vocab);
@@ -313,7 +315,7 @@ extern "C" int rv_topk_select(hipStream_t stream, const float* logits, int rows,
 // exp(v - max) in 64-bit, add up from the left, cut the nucleus at the first prefix that reaches top_p of the
 // total, draw one number from the request's SplitMix64 stream and walk along the weights.  One block a row: all
 // threads sort and weigh, one thread adds and walks (the sums are one after the other by definition).  A row
-// with a candidate that is no number gets -1 and keeps its stream.
+// one of whose own top_k candidates is no finite number gets -1 and keeps its stream, as the host refuses it.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float topk_value_of(unsigned long long key) {
   unsigned int b = (unsigned int)(key >> 32);
@@ -337,7 +339,6 @@ draw_kernel(const float* __restrict__ vals, const int* __restrict__ ids, int k, 
     unsigned long long key = 0ull;  // below every candidate's
     if (j < k) {
       const float v = vals[(size_t)row * k + j] + 0.0f;  // -0 as +0: the two compare equal on the host
-      if (!(fabsf(v) <= 3.402823466e38f)) bad = 1;
       key = topk_key(v, ids[(size_t)row * k + j]);
     }
     keys[j] = key;
@@ -359,11 +360,32 @@ draw_kernel(const float* __restrict__ vals, const int* __restrict__ ids, int k, 
       __syncthreads();
     }
   }
-  const int n = top_k[row] > 0 ? (top_k[row] < k ? top_k[row] : k) : k;
+  // What the row keeps: its own top_k of the sorted candidates (0: all of them); -1 marks a row that decodes
+  // greedily among rows that draw, which keeps one and takes it as the arg-max does.
+  const int own = top_k[row];
+  const bool arg_max = own < 0;
+  const int n = arg_max ? 1 : (own > 0 ? (own < k ? own : k) : k);
   const double top = (double)topk_value_of(keys[0]);
-  for (int j = tid; j < n; j += blockDim.x) weight[j] = exp((double)topk_value_of(keys[j]) - top);
+  for (int j = tid; j < n; j += blockDim.x) {
+    const float v = topk_value_of(keys[j]);
+    // the host refuses a row one of whose own candidates is no finite number; what lies beyond the row's top_k
+    // was selected for another row's sake and is not looked at
+    if (!arg_max && !(fabsf(v) <= 3.402823466e38f)) bad = 1;
+    weight[j] = exp((double)v - top);
+  }
   __syncthreads();
   if (tid != 0) return;
+  if (arg_max) {
+    // the largest logit that is a number (the arg-max skips NaN; equal values go by the lower id, which is the
+    // order of the sort); -1 if all k candidates are NaN
+    int pick = -1;
+    for (int i = 0; i < k && pick < 0; ++i) {
+      const float v = topk_value_of(keys[i]);
+      if (v == v) pick = i;
+    }
+    chosen[row] = pick < 0 ? -1 : (int)(0xFFFFFFFFu - (unsigned int)(keys[pick] & 0xFFFFFFFFull));
+    return;
+  }
   if (bad) {
     chosen[row] = -1;
     return;
@@ -403,7 +425,8 @@ draw_kernel(const float* __restrict__ vals, const int* __restrict__ ids, int k, 
   chosen[row] = (int)(0xFFFFFFFFu - (unsigned int)(keys[pick] & 0xFFFFFFFFull));
 }
 
-// vals, ids [rows, k]: the candidates of topk_select (values times 1/T, any order); top_k [rows] (0: all k),
+// vals, ids [rows, k]: the candidates of topk_select (values times 1/T, any order); top_k [rows] (0: all k; -1: no
+// draw, the arg-max of the candidates, for a greedy request among requests that sample),
 // top_p [rows] (64-bit), rng_state [rows] (each request's stream, moved one draw on), chosen [rows].
 extern "C" int rv_draw(hipStream_t stream, const float* vals, const int* ids, int rows, int k, const int* top_k,
                        const double* top_p, unsigned long long* rng_state, int* chosen) {

@@ -44,6 +44,7 @@ class LLMEngine:
         self.scheduler = Scheduler(runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.max_prefill_chunk,
                                    cfg.max_model_len, on_admit=self._on_admit)
         self.sampler = Sampler(runner.model.spec.vocab_size)
+        self._held_back: list[GenerationResult] = []  # results of a step that failed, handed out by the next one
         self.steps = 0
         self.plans = 0  # plans that ran something; fewer than steps when greedy steps followed one another
         self.tokens_run = 0
@@ -79,8 +80,12 @@ class LLMEngine:
 
     # ---- one step --------------------------------------------------------
     def step(self) -> list[GenerationResult]:
+        """Plans and runs one step; returns the requests that ended in it.  If the step fails (the model, the
+        sampler) the exception goes to the caller after the plan's requests have ended with the reason
+        ``error`` and given their pages back; their results, and those of requests that had ended in this step
+        before, come with the next call, and the requests that were not in the plan go on."""
         plan = self.scheduler.schedule()
-        results = [self._result(r) for r in plan.ended]
+        results, self._held_back = self._held_back + [self._result(r) for r in plan.ended], []
         if not plan.portions:
             return results
         entries = []
@@ -91,20 +96,23 @@ class LLMEngine:
             if p.wants_token:
                 wanting.append(p.request)
         self.plans += 1
-        ahead = self._steps_ahead(plan)
-        if ahead > 1:
-            return results + self._decode_ahead(plan, ahead)
         try:
+            ahead = self._steps_ahead(plan)
+            if ahead > 1:
+                return results + self._decode_ahead(plan, ahead)
             logits = self.runner.step(entries, starts=[p.start for p in plan.portions])
             self.steps += 1
             self.tokens_run += plan.num_tokens
             chosen = self.sampler.sample(logits, [r.params for r in wanting], [r.rng for r in wanting])
         except Exception:
             # The cache may hold this step's tokens while the requests do not count them (the sampler refuses
-            # logits that are not finite, for one): the plan's requests end here, so that nothing is run twice
-            # or a portion further on, and the others go on.
+            # logits that are not finite, for one; steps run ahead have taken pages for tokens that were never
+            # chosen): the plan's requests end here, so that nothing is run twice or a portion further on.
+            self._held_back = results
             for p in plan.portions:
-                self.scheduler.abort(p.request, "error")
+                if p.request.state is not RequestState.FINISHED:
+                    self.scheduler.abort(p.request, "error")
+                    self._held_back.append(self._result(p.request))
             raise
         next_tokens = {r.id: t for r, t in zip(wanting, chosen)}
         finished = self.scheduler.commit(plan, next_tokens)

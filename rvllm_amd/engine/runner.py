@@ -26,7 +26,6 @@ from ..kernels import ops
 from ..models.model import DecoderModel
 from ..models.registry import Architecture, get_architecture, load_config
 from ..parts.base import KVNeed
-from ..parts.linear import set_tiled_weights
 from ..weights.loader import load_tensors, open_model_files, tensor_names
 from ..weights.random_init import random_tensors
 from .batch import BatchBuilder, Portion, StepBatch
@@ -162,7 +161,6 @@ class ModelRunner:
         """Model class by config.json, weights by name from the folder's safetensors."""
         engine_config.validate()
         ops.library()  # fail now, and loudly, if the kernels cannot be built or loaded
-        set_tiled_weights(engine_config.tiled_weights)
         arch, config = load_config(model_dir)
         files = open_model_files(model_dir)
         try:
@@ -170,7 +168,7 @@ class ModelRunner:
             model = DecoderModel(arch.build_spec(config, **arch.locate_tensors(tensor_names(files))))
             tensors = load_tensors(files, model.param_specs(), engine_config.torch_dtype, source=str(model_dir),
                                    ignore=arch.ignored_prefixes)
-            model.bind(tensors, engine_config.device, engine_config.torch_dtype)
+            model.bind(tensors, engine_config.device, engine_config.torch_dtype, engine_config.tiled_weights)
         finally:
             for f in files:
                 f.close()
@@ -181,11 +179,10 @@ class ModelRunner:
         """Random weights made on the device (no folder is written)."""
         engine_config.validate()
         ops.library()
-        set_tiled_weights(engine_config.tiled_weights)
         arch = get_architecture(config.architecture)
         model = DecoderModel(arch.build_spec(config))
         tensors = random_tensors(model.param_specs(), seed, engine_config.device, engine_config.torch_dtype)
-        model.bind(tensors, engine_config.device, engine_config.torch_dtype)
+        model.bind(tensors, engine_config.device, engine_config.torch_dtype, engine_config.tiled_weights)
         return cls(model, engine_config)
 
     # ---- warm-up ------------------------------------------------------

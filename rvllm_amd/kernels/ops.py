@@ -279,6 +279,24 @@ def gated_act(gate_up, activation: str, out: Optional[torch.Tensor] = None, four
     return out
 
 
+def add_bias(x, bias: torch.Tensor) -> torch.Tensor:
+    """x + bias, row by row: in place for a tensor; unreduced ``SlicedSums`` are added up and the bias with
+    them, into a new tensor of the product's type."""
+    _gpu(bias)
+    if isinstance(x, SlicedSums):
+        out = torch.empty((x.rows, x.width), dtype=x.dtype, device=x.device)
+        part, slices = x.data, x.slices
+    else:
+        _gpu(x)
+        _need(x.dim() == 2, "add_bias: a matrix is expected")
+        out, part, slices = x, None, 0
+    rows, width = out.shape
+    _need(bias.shape == (width,) and bias.dtype in _DT, f"add_bias: the bias must hold {width} numbers")
+    _check(library().rv_add_bias(_stream(), _ptr(out), _dt(out), _ptr(part), _c_int(slices), _ptr(bias),
+                                 _c_int(bias.dtype == torch.float32), _c_int(rows), _c_int(width)))
+    return out
+
+
 def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
     _gpu(logits)
     _need(logits.dtype == torch.float32, "softcap: logits must be float32")
@@ -656,8 +674,9 @@ def draw(vals: torch.Tensor, ids: torch.Tensor, top_k: torch.Tensor, top_p: torc
          out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token a row from the candidates ``vals, ids [rows, k]`` of ``topk_select``, drawn on the device as the
     host draws (``sampling.sampler.sample_rows``): ``top_k`` int32 and ``top_p`` float64 a row, ``rng_state`` int64
-    a row, each request's SplitMix64 state, which moves one draw on.  -1 for a row whose candidates are not all
-    numbers."""
+    a row, each request's SplitMix64 state, which moves one draw on.  -1 for a row one of whose own ``top_k``
+    candidates is no finite number.  A row with ``top_k`` -1 draws nothing: it gets the largest candidate that is
+    a number, the lower id among equals, as ``argmax`` gives it."""
     _gpu(vals, ids, top_k, top_p, rng_state, out)
     rows, k = vals.shape
     _need(vals.dtype == torch.float32 and ids.dtype == torch.int32 and ids.shape == vals.shape,

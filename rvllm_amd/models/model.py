@@ -42,9 +42,23 @@ class DecoderModel:
             raise ValueError(f"parts ask for the same tensor twice: {dup}")
         return specs
 
-    def bind(self, tensors: dict[str, torch.Tensor], device, dtype: torch.dtype) -> None:
+    def all_parts(self):
+        """Every part of the model, the blocks and what they hold."""
+        yield self.embedding
+        for block in self.blocks:
+            yield block
+            yield from block.parts()
+        yield self.final_norm
+        yield self.head
+
+    def bind(self, tensors: dict[str, torch.Tensor], device, dtype: torch.dtype, tiled_weights: bool = True) -> None:
+        """``tiled_weights``: whether the parts keep their bf16 matrices a second time in tiles for the
+        few-row product (``EngineConfig.tiled_weights``); each model carries its own setting."""
         self.device = torch.device(device)
         self.dtype = dtype
+        self.tiled_weights = bool(tiled_weights)
+        for part in self.all_parts():
+            part.tiled_weights = self.tiled_weights
         self.embedding.bind(tensors, self.spec.prefix, self.device, dtype)
         for layer, block in zip(self.spec.layers, self.blocks):
             block.bind(tensors, layer.prefix, self.device, dtype)

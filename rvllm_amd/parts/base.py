@@ -44,6 +44,9 @@ class Part:
     and steps of a model that holds such a part are never taken from a graph."""
 
     capturable: bool = True
+    # Whether the part lays bf16 matrices out in tiles for the few-row product (``linear.decode_weight``): the
+    # engine's setting, which the model writes into every part it holds before it binds them.
+    tiled_weights: bool = True
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
         return []

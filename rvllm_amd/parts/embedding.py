@@ -70,9 +70,10 @@ class LMHead(Head):
 
     def bind(self, tensors, prefix, device, dtype) -> None:
         if self.tied:
-            self.weight = decode_weight(self.embedding.table)  # the table itself stays row by row for the lookup
+            self.weight = decode_weight(self.embedding.table, self.tiled_weights)  # the table itself stays row by row for the lookup
         else:
-            self.weight = decode_weight(tensors[self.weight_name].to(device=device, dtype=dtype).contiguous())
+            self.weight = decode_weight(tensors[self.weight_name].to(device=device, dtype=dtype).contiguous(),
+                                        self.tiled_weights)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = linear(x, self.weight, out_dtype=torch.float32)

@@ -17,22 +17,37 @@ import torch
 from ..kernels import ops
 
 
-# Whether ``decode_weight`` lays bf16 matrices out in tiles for the few-row product (the engine's setting; the
-# matrix row by row is kept beside the tiles for the products that go to the library).
-_TILED_WEIGHTS = True
-
-
-def set_tiled_weights(on: bool) -> None:
-    global _TILED_WEIGHTS
-    _TILED_WEIGHTS = bool(on)
-
-
-def decode_weight(w: torch.Tensor):
-    """A part's matrix ``[N, K]`` as its products want it: bf16 on the GPU in tiles (``ops.TiledWeight``, the
-    rows kept beside them), anything else as it is."""
-    if _TILED_WEIGHTS and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2:
+def decode_weight(w: torch.Tensor, tiled: bool = True):
+    """A part's matrix ``[N, K]`` as its products want it: with ``tiled`` (the part's ``tiled_weights``, which
+    is the engine's setting) a bf16 matrix on the GPU goes into tiles for the few-row product
+    (``ops.TiledWeight``; the matrix row by row is kept beside the tiles for the products that go to the
+    library), anything else stays as it is."""
+    if tiled and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2:
         return ops.TiledWeight(w.contiguous())
     return w
+
+
+def tensor_names(defaults: dict, given) -> dict:
+    """A part's table of tensor names: ``defaults`` (role -> name under the layer's prefix, without
+    ``.weight``) with the roles that the part's spec names otherwise (``names``) laid over it."""
+    names = dict(defaults)
+    for role, name in dict(given or {}).items():
+        names[str(role)] = str(name)
+    return names
+
+
+def bias_roles(given, roles) -> frozenset:
+    """The roles among ``roles`` whose projection has a bias: the spec's ``bias`` is absent or False (none),
+    True (all of them) or a list of roles."""
+    if not given:
+        return frozenset()
+    if given is True:
+        return frozenset(roles)
+    wanted = frozenset(str(r) for r in given)
+    unknown = wanted - frozenset(roles)
+    if unknown:
+        raise ValueError(f"bias for unknown projections {sorted(unknown)}; this part has {sorted(roles)}")
+    return wanted
 
 
 def linear(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,

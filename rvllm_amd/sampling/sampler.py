@@ -131,8 +131,10 @@ class DeviceDraws:
     ``topk_select`` and then ``ops.draw``, which does what ``sample_rows`` does with each request's stream of
     numbers kept on the device.  The device selects as many candidates for every row as the row that asks for
     most; a row keeps its own ``top_k`` of them after the sort, which are the ones it would have had selected
-    (equal values go by the lower id both times), and rows that decode greedily keep one.  A row whose largest
-    logits are not all numbers gets -1 (the arg-max skips such logits, the host's draw refuses them)."""
+    (equal values go by the lower id both times).  A row that samples gets -1 if one of its own ``top_k``
+    largest logits is no finite number, as the host's draw refuses it; what was selected beyond them for another
+    row's sake is not looked at.  A row that decodes greedily takes the largest candidate that is a number, as
+    the arg-max does (``top_k`` -1 tells the kernel so), and draws no number from its stream."""
 
     def __init__(self, vocab_size: int, params: Sequence[SamplingParams], rngs: Sequence[SplitMix64], device):
         ks = [p.kernel_k(vocab_size) for p in params if not p.is_greedy()]
@@ -142,7 +144,7 @@ class DeviceDraws:
         greedy = [p.is_greedy() for p in params]
         self.inv_temp = torch.tensor([1.0 if g else 1.0 / p.temperature for p, g in zip(params, greedy)],
                                      dtype=torch.float32, device=device)
-        self.top_k = torch.tensor([1 if g else p.top_k for p, g in zip(params, greedy)], dtype=torch.int32,
+        self.top_k = torch.tensor([-1 if g else p.top_k for p, g in zip(params, greedy)], dtype=torch.int32,
                                   device=device)
         self.top_p = torch.tensor([1.0 if g else p.top_p for p, g in zip(params, greedy)], dtype=torch.float64,
                                   device=device)

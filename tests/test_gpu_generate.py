@@ -264,8 +264,27 @@ def test_greedy_steps_ahead_change_no_token(model_dirs, name):
     def run(ahead, tight, places=4):
         engine = LLMEngine.from_model_dir(model_dirs[name], EngineConfig(
             dtype="bfloat16", max_model_len=200, max_num_seqs=places, max_num_batched_tokens=64, max_prefill_chunk=64,
-            max_cache_tokens=160 if tight else 800, greedy_steps_ahead=ahead))
+            max_cache_tokens=112 if tight else 800, greedy_steps_ahead=ahead))
         vocab = engine.runner.model.spec.vocab_size
+        params_of = {}
+        engine.draws = []  # every step whose tokens the device drew: (request ids, logits, streams before, tokens)
+        decode_ahead = engine.runner.decode_ahead
+
+        def watched(entries, steps, choose=None):
+            if choose is None:
+                return decode_ahead(entries, steps, None)
+
+            def recording(logits, out):
+                before = choose.state.clone()
+                choose(logits, out)
+                engine.draws.append(([rid for rid, _ in entries], logits.clone(), before.cpu().tolist(), out.clone()))
+                return out
+
+            return decode_ahead(entries, steps, recording)
+
+        engine.runner.decode_ahead = watched
+        engine.params_of = params_of
+        engine.set_backs = 0
         prompts = [[(11 * i + j) % vocab for i in range(n)] for j, n in enumerate((5, 18, 33, 9))]
         out = {}
         sampling = {"all greedy": {}, "one samples": {2: SamplingParams(0.9, 20, 1.0, seed=3)},
@@ -276,11 +295,13 @@ def test_greedy_steps_ahead_change_no_token(model_dirs, name):
             before = engine.plans, engine.steps
             for j, prompt in enumerate(prompts):
                 params = sampled.get(j, SamplingParams())
+                params_of[(phase, j)] = params
                 engine.add_request((phase, j), prompt, params, max_new_tokens=(37, 50, 23, 44)[j],
                                    eos_ids=run.eos if j == 1 else (), ignore_eos=False)
             while engine.has_work():
                 for res in engine.step():
                     out[res.request_id] = (res.tokens, res.finish_reason)
+                    engine.set_backs += res.set_backs
             run.planned[(ahead, tight, places, phase)] = (engine.plans - before[0], engine.steps - before[1])
         return out, engine
 
@@ -315,6 +336,19 @@ def test_greedy_steps_ahead_change_no_token(model_dirs, name):
     for out in (tight_single, tight_ahead, few_single, few_ahead):  # and the others ran to their ends
         assert {key: (len(tokens), reason) for key, (tokens, reason) in out.items()} == \
                {key: (len(tokens), reason) for key, (tokens, reason) in single.items()}
+    # The requests that sample, in exactly these runs: every token that the device drew, with requests set back
+    # or waiting around it, is the token that the host's sampler draws from the same logits with the request's
+    # stream as it stood before the draw; and a greedy request's among them is the arg-max's.
+    from rvllm_amd.sampling.sampler import Sampler, SplitMix64
+
+    for engine in (e4, t4, f4):
+        assert len(engine.draws) > 30
+        sampler = Sampler(engine.runner.model.spec.vocab_size)
+        for rids, logits, states, tokens in engine.draws:
+            params = [engine.params_of[rid] for rid in rids]
+            rngs = [SplitMix64(state) for state in states]
+            assert sampler.sample(logits, params, rngs) == tokens.cpu().tolist()
+    assert t4.set_backs >= 1 and t1.set_backs >= 1 and e4.set_backs == 0  # the tight runs did set requests back
 
 
 def test_eos_and_capacity_reasons(model_dirs):

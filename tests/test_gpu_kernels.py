@@ -886,6 +886,32 @@ def test_the_draw_on_the_device_is_the_hosts(k):
     assert got[0] == -1 and all(t >= 0 for t in got[1:]) and state[0] == before[0] and (state[1:] != before[1:]).all()
 
 
+def test_the_draw_looks_at_a_rows_own_candidates_only():
+    """In a batch the device selects for every row as many candidates as the row that asks for most.  Whether a
+    row has a token must not depend on who else is in the batch: a row that keeps 3 is judged by its 3 largest
+    (a -inf beyond them is nobody's business, one among them is refused as the host refuses it), and a row
+    that decodes greedily takes the largest candidate that is a number, as the arg-max does."""
+    from rvllm_amd.sampling.sampler import SplitMix64, sample_rows
+
+    k = 8
+    vals = torch.tensor([[5.0, 1.0, 3.0, 2.0, float("-inf"), 0.5, 4.0, -1.0],   # keeps 3: -inf lies beyond
+                         [5.0, 1.0, float("-inf"), 2.0, 0.0, 0.5, 4.0, -1.0],   # keeps all 8: -inf is among them
+                         [float("nan"), 1.0, 7.0, 7.0, 0.0, 0.5, 4.0, -1.0],    # greedy: NaN skipped, 7 twice
+                         [float("nan")] * 8,                                    # greedy: nothing is a number
+                         [2.0, float("inf"), 3.0, 2.0, 1.0, 0.5, 4.0, -1.0]])   # greedy: +inf is the largest
+    ids = torch.tensor([[10, 11, 12, 13, 14, 15, 16, 17]] * 5, dtype=torch.int32)
+    ids[2] = torch.tensor([3, 4, 9, 6, 5, 7, 8, 2])  # the two 7s have ids 9 and 6: the lower one
+    top_k = torch.tensor([3, 0, -1, -1, -1], dtype=torch.int32)
+    top_p = torch.tensor([1.0] * 5, dtype=torch.float64)
+    seeds = [11, 12, 13, 14, 15]
+    state = dev(torch.tensor(seeds, dtype=torch.int64))
+    got = ops.draw(dev(vals), dev(ids), dev(top_k), dev(top_p), state).cpu().tolist()
+    want0 = sample_rows(vals[:1, [0, 6, 2]].numpy(), ids[:1, [0, 6, 2]].numpy(), [3], [1.0], [SplitMix64(11)], 100)[0]
+    assert got == [want0, -1, 6, -1, 11]
+    after = state.cpu().tolist()
+    assert after[0] != 11 and after[1:] == seeds[1:]  # only the row that drew moved its stream
+
+
 def test_kernels_refuse_what_they_cannot_do():
     x = torch.randn(4, 32)
     with pytest.raises(ops.KernelError, match="GPU"):

@@ -240,3 +240,120 @@ def test_a_requests_tokens_from_a_place_on():
     for start in range(7):
         for count in range(1, 8 - start):
             assert req.tokens_at(start, count) == req.tokens[start:start + count], (start, count)
+
+
+# ---- the engine's loop around a step that fails -----------------------------------------------------------
+class FailingRunner:
+    """What ``LLMEngine`` asks of a runner, without a GPU: the cache's books are kept as the real step keeps
+    them; a step that holds a token of ``poison`` extends the cache and then raises, as a kernel error or a
+    sampler that meets logits that are no numbers would.  Its 'logits' are the next tokens themselves."""
+
+    def __init__(self, cache, config, poison):
+        import types
+
+        self.cache, self.config, self.poison, self.device = cache, config, poison, "cpu"
+        self.model = types.SimpleNamespace(spec=types.SimpleNamespace(vocab_size=VOCAB))
+        self.storage = types.SimpleNamespace(clear_slot=lambda slot: None)
+        self.seen = {}
+
+    def step(self, entries, starts=None):
+        self.cache.extend_all([(rid, self.cache.length(rid) + len(toks)) for rid, toks, _ in entries])
+        if any(self.poison in toks for _, toks, _ in entries):
+            raise RuntimeError("the step failed")
+        out = []
+        for rid, toks, want in entries:
+            start = self.cache.length(rid)
+            self.seen[rid] = (self.seen[rid] if start else []) + list(toks)
+            self.cache.commit(rid, start + len(toks))
+            if want:
+                out.append(next_token(self.seen[rid]))
+        return out
+
+
+    def decode_ahead(self, entries, steps, choose=None):
+        """Several decode steps from one plan: pages for all of them are taken first, as the real runner does."""
+        self.cache.extend_all([(rid, self.cache.length(rid) + steps) for rid, _ in entries])
+        if any(token == self.poison for _, token in entries):
+            raise RuntimeError("the steps ahead failed")
+        rows = []
+        tokens = [token for _, token in entries]
+        for _ in range(steps):
+            for (rid, _), token in zip(entries, tokens):
+                self.seen[rid].append(token)
+            tokens = [next_token(self.seen[rid]) for rid, _ in entries]
+            rows.append(tokens)
+        for rid, _ in entries:
+            self.cache.commit(rid, self.cache.length(rid) + steps)
+        return rows
+
+
+class PassThroughSampler:
+    vocab_size = VOCAB
+
+    def sample(self, logits, params, rngs):
+        return list(logits)
+
+
+def test_a_step_that_fails_ends_its_requests_and_the_others_go_on():
+    import types
+
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.engine.engine import LLMEngine
+
+    cache = CacheManager([KVNeed(1, 8, 8), KVNeed(1, 8, None)], 4, 64, 4)
+    config = EngineConfig(max_model_len=256, max_num_seqs=2, max_num_batched_tokens=16, max_prefill_chunk=8,
+                          greedy_steps_ahead=1, page_size=16)
+    free_at_first = dict(cache.free_pages())
+    engine = LLMEngine(FailingRunner(cache, config, poison=90))
+    engine.sampler = PassThroughSampler()
+    good, bad, late = [1, 2, 3], [4, 5, 90, 6], [7, 8, 9, 10, 11]
+    engine.add_request("good", good, max_new_tokens=1)
+    engine.add_request("bad", bad, max_new_tokens=4)
+    engine.add_request("late", late, max_new_tokens=3)  # waits: two places only
+    # the first step holds both prompts; "good" would end in it (one new token), "bad" makes it fail
+    with pytest.raises(RuntimeError, match="the step failed"):
+        engine.step()
+    assert not cache.has_request("good") and not cache.has_request("bad")  # their pages are back
+    assert cache.free_pages() == free_at_first
+    done = {}
+    while engine.has_work():
+        for res in engine.step():
+            done[res.request_id] = res
+    assert done["good"].finish_reason == "error" and done["bad"].finish_reason == "error"
+    assert done["good"].tokens == [] and done["bad"].tokens == []
+    assert done["late"].finish_reason == "length" and done["late"].tokens == expected_output(late, 3)
+    assert cache.free_pages() == free_at_first
+    cache.check()
+    # nothing is handed out twice
+    assert engine.step() == []
+
+
+def test_steps_ahead_that_fail_end_their_requests_too():
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.engine.engine import LLMEngine
+
+    cache = CacheManager([KVNeed(1, 8, 8), KVNeed(1, 8, None)], 4, 64, 4)
+    config = EngineConfig(max_model_len=256, max_num_seqs=2, max_num_batched_tokens=16, max_prefill_chunk=8,
+                          greedy_steps_ahead=4, page_size=16)
+    free_at_first = dict(cache.free_pages())
+    prompt, other = [2, 5, 6], [9, 8, 7, 6]
+    poison = expected_output(prompt, 6)[4]  # the fifth new token, which the second plan of steps ahead starts from
+    assert poison not in expected_output(prompt, 4) and poison not in expected_output(other, 12) + prompt + other
+    engine = LLMEngine(FailingRunner(cache, config, poison))
+    engine.sampler = PassThroughSampler()
+    engine.add_request("a", prompt, max_new_tokens=12)
+    engine.add_request("late", other, max_new_tokens=3)
+    engine.scheduler.max_num_seqs = 1  # "late" waits until "a" is gone; nobody waits for a place that is free
+    with pytest.raises(RuntimeError, match="the steps ahead failed"):
+        while engine.has_work():
+            assert engine.step() == []
+    assert engine.plans < engine.steps  # steps ahead did run before
+    assert not cache.has_request("a") and cache.free_pages() == free_at_first
+    engine.scheduler.max_num_seqs = 2
+    done = {}
+    while engine.has_work():
+        for res in engine.step():
+            done[res.request_id] = res
+    assert done["a"].finish_reason == "error" and done["a"].tokens == expected_output(prompt, 5)
+    assert done["late"].tokens == expected_output(other, 3)
+    cache.check()
