@@ -424,16 +424,26 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
 
 MFMA_ATTENTION_MAX_HEAD_DIM = 256
 MFMA_ATTENTION_MAX_GROUP = 16
-# What the split plan of the decode kernel knows about the machine (measured on MI355X with keys and values of
-# 256 per head; microseconds): the kernel runs one wave a SIMD, 1024 at once on 256 CUs; a wave takes about 3.2
-# for a block of 32 keys when it waits for nobody; 1024 waves together stream about 6.3 TB/s; launches, the first
-# reads and the merge cost about 10.6 (7 without a merge), and the merge 0.1 more per split.
-_ATTN_WAVE_SLOTS = 1024
-_ATTN_BLOCK_US = 3.2
+# What the split plan of the decode kernel knows about the machine (measured on MI355X at head sizes 64, 128 and
+# 256; microseconds): how many of the kernel's waves the machine holds at once is the library's answer for the
+# head size at hand (what the kernel's registers allow: one wave a SIMD, 1024 in all, at head size 256; two at
+# 128; four at 64); a wave that waits for nobody takes about 1 + head size / 100 for a block of 32 keys (3.6 at
+# 256, 2.3 at 128); the waves together stream about 6.3 TB/s; launches and the first reads cost about 7, and the
+# merge 0.1 more per split.
+_ATTN_WAVE_SLOTS_FALLBACK = 1024
+_ATTN_BLOCK_US = (1.0, 0.01)  # a + b * head size
 _ATTN_BYTES_PER_US = 6.3e6
-_ATTN_FIXED_US = 10.6
+_ATTN_FIXED_US = 7.0
 _ATTN_FIXED_UNSPLIT_US = 7.0
 _ATTN_MERGE_US_PER_SPLIT = 0.1
+
+
+@functools.lru_cache(maxsize=None)
+def attention_wave_slots(head_dim: int) -> int:
+    """How many waves of the matrix-core decode kernel for this head size the GPU holds at once."""
+    entry = getattr(library(), f"rv_attn_mfma_wave_slots_g{(head_dim // 16 - 1) // 4}", None)
+    slots = entry(_c_int(head_dim)) if entry is not None else -1
+    return slots if slots > 0 else _ATTN_WAVE_SLOTS_FALLBACK
 
 
 def mfma_attention_covers(k_pages: torch.Tensor, v_pages: torch.Tensor, num_q_heads: int) -> bool:
@@ -444,17 +454,19 @@ def mfma_attention_covers(k_pages: torch.Tensor, v_pages: torch.Tensor, num_q_he
 
 @functools.lru_cache(maxsize=4096)
 def plan_attention_splits(num_requests: int, max_portion: int, max_context: int, nkv: int, group: int,
-                          window: Optional[int], head_dim: int = 256) -> tuple[int, int, int]:
+                          window: Optional[int], head_dim: int = 256,
+                          wave_slots: int = _ATTN_WAVE_SLOTS_FALLBACK) -> tuple[int, int, int]:
     """(tiles per request, number of key splits, keys per split) for the
     matrix-core decode kernel.  A tile is 16 / group_pad tokens of one request
     and one key/value head; its keys are split over waves.
 
     The number of splits is the one a small model of the machine likes best:
-    the waves run in rounds of 1024 (one a SIMD); a round takes what its
-    longest wave takes alone or what its bytes take at full streaming rate,
-    whichever is longer; a last round that is not full still takes a wave's
-    whole time, which is why 1.3 rounds are worse than 1 or 2; every split
-    adds to the merge."""
+    the waves run in rounds of ``wave_slots`` (``attention_wave_slots``: as
+    many as the machine holds at once); a round takes what its longest wave
+    takes alone or what its bytes take at full streaming rate, whichever is
+    longer; a last round that is not full still takes a wave's whole time,
+    which is why 1.3 rounds are worse than 1 or 2; every split adds to the
+    merge."""
     group_pad = 1
     while group_pad < group:
         group_pad *= 2
@@ -467,17 +479,18 @@ def plan_attention_splits(num_requests: int, max_portion: int, max_context: int,
     blocks = -(-span // 32)
     units = num_requests * tiles * nkv
     block_bytes = 32 * head_dim * 2 * 2  # keys and values of a block, bf16
+    block_us = _ATTN_BLOCK_US[0] + _ATTN_BLOCK_US[1] * head_dim
     best = None
     for splits in range(1, min(blocks, 512) + 1):
         per = -(-blocks // splits)  # blocks a split
         if per * (splits - 1) >= blocks:
             continue  # the last split would be empty: the same plan as with fewer splits
         waves = units * splits
-        full_rounds, rest = divmod(waves, _ATTN_WAVE_SLOTS)
-        alone = per * _ATTN_BLOCK_US
-        time = full_rounds * max(alone, _ATTN_WAVE_SLOTS * per * block_bytes / _ATTN_BYTES_PER_US)
+        full_rounds, rest = divmod(waves, wave_slots)
+        alone = per * block_us
+        time = full_rounds * max(alone, wave_slots * per * block_bytes / _ATTN_BYTES_PER_US)
         if rest:  # fewer waves draw less than the full rate: about its square root of their share
-            rate = _ATTN_BYTES_PER_US * (rest / _ATTN_WAVE_SLOTS) ** 0.5
+            rate = _ATTN_BYTES_PER_US * (rest / wave_slots) ** 0.5
             time += max(alone, rest * per * block_bytes / rate)
         time += _ATTN_FIXED_US + _ATTN_MERGE_US_PER_SPLIT * splits if splits > 1 else _ATTN_FIXED_UNSPLIT_US
         if best is None or time < best[0] * (1.0 - 1e-9):
@@ -526,14 +539,128 @@ def plan_attention_in_block(max_portion: int, max_context: int, group: int, wind
 PREFILL_MIN_PORTION = 16
 
 
+# The prompt kernel's long tiles in pieces (``plan_prefill_pieces``), as measured on MI355X (microseconds): a
+# block walks a block of 64 keys in 0.85 + head size / 400 (1.5 at 256) and has a fixed cost of some nine such
+# blocks (its queries and table read, the first keys waited for, its sums written); merging costs a launch and
+# the pieces' sums written and read again.  Pieces are taken where they shorten the launch by a tenth at least.
+_PREFILL_BLOCK_US = (0.85, 1.0 / 400.0)
+_PREFILL_PIECE_FIXED = 9.0
+_PREFILL_MERGE_US = 6.0
+_PREFILL_BYTES_PER_US = 5.0e6
+_PREFILL_PIECES_GAIN = 1.1
+_PREFILL_PIECES_MOST = 32
+_PREFILL_PIECE_LEAST = 2  # blocks of keys
+_PREFILL_CUT_BELOW = 4    # tiles are cut only while they are fewer than a quarter of the blocks the machine holds
+
+
+@functools.lru_cache(maxsize=None)
+def attention_prefill_block_slots(head_dim: int) -> int:
+    """How many blocks of the prompt attention kernel for this head size the GPU holds at once."""
+    entry = getattr(library(), f"rv_attn_prefill_block_slots_g{(head_dim // 16 - 1) // 4}", None)
+    slots = entry(_c_int(head_dim)) if entry is not None else -1
+    return slots if slots > 0 else 256
+
+
+def plan_prefill_pieces(lengths, starts, tokens_per_tile: int, window: Optional[int], portion_min: int,
+                        head_dim: int, nkv: int, block_slots: int = 256) -> tuple[int, int]:
+    """(blocks of 64 keys a piece at most, pieces a tile at most) for the prompt kernel in this step; (any, 1)
+    means a tile a block.  ``lengths`` and ``starts``: the portions' tokens and first positions;
+    ``block_slots``: the kernel's blocks that the machine holds at once.
+
+    A tile (``tokens_per_tile`` tokens of a portion) walks the keys its tokens see in blocks of 64.  While the
+    blocks all fit the machine at once, a launch lasts as long as its longest block; beyond, as the blocks'
+    work spread over the machine and half a longest block for the uneven end.  Cutting the long tiles shortens
+    the longest block, adds blocks with their fixed cost and the merge: it pays where few tiles walk many keys
+    (a portion of a hundred tokens deep in a long context: 16 blocks for 256 CUs), not where the tiles fill
+    the machine already (a prompt of 2 048 tokens in one portion is as many tiles as there are CUs, and cut
+    tiles would wait for a second turn).  The cut that makes the launch shortest by this count is taken."""
+    import numpy as np
+
+    whole = (1 << 20, 1)
+    lengths = np.asarray(lengths, dtype=np.int64)
+    starts = np.asarray(starts, dtype=np.int64)
+    taken = lengths >= portion_min
+    if not taken.any():
+        return whole
+    lengths, starts = lengths[taken], starts[taken]
+    tiles = -(-lengths // tokens_per_tile)
+    of = np.repeat(np.arange(len(lengths)), tiles)  # the request of every tile
+    first = np.zeros(len(lengths), dtype=np.int64)
+    np.cumsum(tiles[:-1], out=first[1:])
+    tok0 = (np.arange(int(tiles.sum())) - first[of]) * tokens_per_tile
+    ntok = np.minimum(tokens_per_tile, lengths[of] - tok0)
+    p_first = starts[of] + tok0
+    kmin = np.maximum(0, p_first - window + 1) if window else np.zeros_like(p_first)
+    cost = -(-(p_first + ntok - (kmin & ~31)) // 64)
+    total, longest = int(cost.sum()), int(cost.max())
+    block_us = _PREFILL_BLOCK_US[0] + _PREFILL_BLOCK_US[1] * head_dim
+    if len(cost) * nkv * _PREFILL_CUT_BELOW > block_slots:
+        return whole  # measured: where the tiles fill a quarter of the machine or more, pieces gain little or lose
+
+    def launch(piece_max):
+        pieces = -(-cost // piece_max)
+        blocks = int(pieces.sum()) * nkv
+        long_one = -(-longest // -(-longest // piece_max)) + _PREFILL_PIECE_FIXED  # the longest tile's pieces are equal
+        if blocks <= block_slots:
+            time = long_one * block_us
+        else:
+            time = ((total * nkv + blocks * _PREFILL_PIECE_FIXED) / block_slots + 0.5 * long_one) * block_us
+        cut = int(pieces[pieces > 1].sum())
+        if cut:
+            time += _PREFILL_MERGE_US + cut * nkv * 2 * 64 * head_dim * 4 / _PREFILL_BYTES_PER_US
+        return time
+
+    best = (launch(longest), longest, 1)
+    for pieces in range(2, _PREFILL_PIECES_MOST + 1):
+        piece_max = -(-longest // pieces)
+        if piece_max < _PREFILL_PIECE_LEAST:
+            break
+        time = launch(piece_max)
+        if time < best[0]:
+            best = (time, piece_max, -(-longest // piece_max))
+    if best[2] > 1 and launch(longest) >= _PREFILL_PIECES_GAIN * best[0]:
+        return best[1], best[2]
+    return whole
+
+
+def _prefill_pieces(step, window, tokens_per_tile, tiles, portion_min, hd, nkv, device, forced):
+    """(piece_max, pieces_max, room for the pieces' sums) for the prompt kernel in this step; made once a step
+    for the layers that agree in window and sizes (``step.shared``).  ``forced``: (piece_max, pieces_max)."""
+    shared = getattr(step, "shared", None)
+    key = ("prefill_pieces", window, tokens_per_tile, tiles, portion_min, hd, nkv, forced)
+    if shared is not None and key in shared:
+        return shared[key]
+    piece_max, pieces_max = 1 << 20, 1
+    if forced is not None:
+        piece_max, pieces_max = forced
+    else:
+        starts = getattr(step, "host_q_start", None)
+        first = getattr(step, "host_chunk_start", None)
+        if starts is not None and first is not None:
+            lengths = [int(starts[i + 1] - starts[i]) for i in range(step.num_requests)]
+            piece_max, pieces_max = plan_prefill_pieces(lengths, first, tokens_per_tile, window, portion_min, hd, nkv,
+                                                        attention_prefill_block_slots(hd))
+    part = None
+    if pieces_max > 1:
+        part = torch.empty(step.num_requests * tiles * nkv * pieces_max * (64 * hd + 128), dtype=torch.float32,
+                           device=device)
+    result = (int(piece_max), int(pieces_max), part)
+    if shared is not None:
+        shared[key] = result
+    return result
+
+
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                          step, out: torch.Tensor, num_q_heads: int, scale: float, window: Optional[int],
                          splits: Optional[tuple[int, int]] = None, prefill_kernel: Optional[bool] = None,
-                         in_block: Optional[bool] = None) -> torch.Tensor:
+                         in_block: Optional[bool] = None,
+                         prefill_pieces: Optional[tuple[int, int]] = None) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``splits`` = (number, keys per
-    split) overrides the plan, ``prefill_kernel`` the choice of kernel and
-    ``in_block`` whether a tile's splits are merged inside one block (tests
-    use them to force every path)."""
+    split) overrides the plan, ``prefill_kernel`` the choice of kernel,
+    ``in_block`` whether a tile's splits are merged inside one block and
+    ``prefill_pieces`` = (blocks of 64 keys a piece at most, pieces a tile at
+    most) how the prompt kernel cuts its long tiles (tests use them to force
+    every path)."""
     _gpu(q, k_pages, v_pages, block_table, out)
     _i32(block_table)
     n = q.shape[0]
@@ -573,14 +700,17 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     if use_prefill:
         tokens_per_block = 64 // group_pad
         tiles = -(-longest // tokens_per_block)
+        piece_max, pieces_max, part = _prefill_pieces(step, window, tokens_per_block, tiles, portion_min, hd, nkv,
+                                                      q.device, prefill_pieces)
         entry = getattr(lib, f"rv_attn_prefill_{suffix}")
         _check(entry(_stream(), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
                      _c_int(block_table.shape[1]), _ptr(step.q_start), _ptr(step.chunk_start), _ptr(out), _c_int(n),
                      _c_int(step.num_requests), _c_int(tiles), _c_int(num_q_heads), _c_int(nkv), _c_int(hd),
-                     _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_int(portion_min), _c_float(scale)))
+                     _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_int(portion_min), _c_float(scale),
+                     _c_int(piece_max), _c_int(pieces_max), _ptr(part)))
     if shortest_rest > 0:
         tiles, num_splits, split_len = plan_attention_splits(step.num_requests, shortest_rest, step.max_context, nkv,
-                                                             group, window, hd)
+                                                             group, window, hd, attention_wave_slots(hd))
         block_cols = 0
         merged = None
         if in_block is not False:

@@ -702,6 +702,70 @@ def test_shared_tiles_attention_missing_page_shows():
     assert torch.isnan(got[32:]).all() and not torch.isnan(got[:32]).any()
 
 
+@pytest.mark.parametrize("nq,nkv,hd", [(8, 4, 256), (32, 16, 128), (6, 1, 48), (5, 5, 240)])
+@pytest.mark.parametrize("pieces", [(1, 5), (2, 3), (3, 2), (4, 64), (1, 2)])
+def test_prompt_attention_with_long_tiles_in_pieces(nq, nkv, hd, pieces):
+    """The prompt kernel with its long tiles cut into pieces, a block each, merged afterwards: pieces of a single
+    block of keys, pieces that leave some tiles whole, more pieces allowed than any tile has, fewer than the
+    piece length asks for (the pieces are then longer); portions from position 0, continuing ones, short ones
+    among them, with and without a window.  The same as a tile a block, and as the 64-bit reference."""
+    for portions, window in (([(0, 300)], None), ([(257, 130), (0, 70), (40, 17)], None), ([(0, 300), (5, 2)], 64),
+                             ([(990, 100)], 1024), ([(100, 257), (3, 1), (0, 33)], 100)):
+        case = Case(portions, nq, nkv, hd, 16, torch.bfloat16, 31, window)
+        want = case.reference(hd ** -0.5).float()
+        got = case.run("mfma", hd ** -0.5, prefill_pieces=pieces).float()
+        assert torch.allclose(got, want, **tol(torch.bfloat16)), (portions, window)
+        whole = case.run("mfma", hd ** -0.5, prefill_pieces=(1 << 20, 1)).float()
+        assert torch.allclose(got, whole, **tol(torch.bfloat16)), (portions, window)
+
+
+def test_prompt_attention_cuts_its_tiles_where_few_walk_many_keys():
+    """The choice: a short portion deep in a long context (a prompt that arrives in portions of 128 tokens: four
+    tiles a key/value head that walk 8 000 keys each, on a machine of 256 CUs) has its tiles cut into pieces;
+    a whole prompt of 2 048 tokens is bound by all its blocks of keys together, not by its longest tile, and
+    is left a tile a block, as are portions that fill the machine, short ones and decoded tokens."""
+    plan = lambda lengths, starts, window=None: ops.plan_prefill_pieces(lengths, starts, 32, window, 16, 256, 4)
+    assert plan([128], [8000])[1] > 4
+    assert plan([64], [8000], window=1024)[1] > 1    # under the window its tiles see 1 087 keys: 8 blocks for 256 CUs
+    assert plan([2048], [0])[1] == 1
+    assert plan([1024], [0])[1] == 1
+    assert plan([2048] * 4, [30000] * 4)[1] == 1
+    assert plan([64] * 8, [0] * 8)[1] == 1
+    assert plan([1] * 8, [500] * 8)[1] == 1          # left to the other kernel
+    piece_max, pieces_max = plan([128], [30000])
+    assert piece_max >= 8 and pieces_max * piece_max >= -(-30128 // 64)  # the pieces cover the longest tile
+    # through the kernel, with the plan it makes for itself, at sizes where it cuts
+    case = Case([(4000, 100), (700, 1)], 8, 4, 256, 16, torch.bfloat16, 32, None)
+    assert ops.plan_prefill_pieces([100, 1], [4000, 700], 32, None, 16, 256, 4)[1] > 1
+    want = case.reference(1.0 / 16).float()
+    assert torch.allclose(case.run("mfma", 1.0 / 16).float(), want, **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("far", [0, 17, 63, 64, 200, 255])
+def test_prompt_attention_in_pieces_finds_one_key(far):
+    """One key carries all the weight, wherever it lies among pieces of two blocks of keys: the piece that holds
+    it must win the merge for every later token, and no piece of an earlier token may see it; a page that is
+    missing shows in exactly the tokens that see it."""
+    nq, nkv, hd, n = 4, 2, 64, 256
+    for window in (None, 40):
+        case = Case([(0, n)], nq, nkv, hd, 16, torch.bfloat16, 14, window, drop_passed_pages=False)
+        case.k_all[0] *= 0.01
+        case.k_log *= 0.01
+        _plant(case, 0, far, 1, 5, 40.0)
+        case.q[:] = 0
+        case.q[:, :, 5] = 40.0
+        got = case.run("mfma", 1.0, prefill_kernel=True, prefill_pieces=(2, 2)).float()
+        assert torch.allclose(got, case.reference(1.0).float(), **tol(torch.bfloat16))
+        v_far = case.v_all[0][far, 1].float()
+        for t in (far, min(far + 39, n - 1), min(far + 40, n - 1), n - 1):
+            sees = t >= far and (window is None or t - far < window)
+            assert torch.allclose(got[t, 2:], v_far.expand(2, hd), atol=2e-2) == sees, (far, window, t)
+    case = Case([(0, 200)], 2, 1, 32, 16, torch.bfloat16, 16)
+    case.table[0, 2] = -1  # keys 32..47 are gone
+    got = case.run("mfma", 1.0, prefill_kernel=True, prefill_pieces=(1, 4))
+    assert torch.isnan(got[32:]).all() and not torch.isnan(got[:32]).any()
+
+
 @pytest.mark.parametrize("splits", [(1, 224), (2, 128), (7, 32), (4, 64)])
 @pytest.mark.parametrize("window", [None, 100])
 def test_paged_attention_mfma_every_split(splits, window):

@@ -142,7 +142,8 @@ def test_decode_attention_under_its_own_plan_at_long_contexts(nq, nkv, hd, conte
     want = case.reference(scale)
     ok, why = close(case.run(scale), want)
     assert ok, why
-    tiles, splits, split_len = ops.plan_attention_splits(batch, 1, context, nkv, nq // nkv, window, hd)
+    tiles, splits, split_len = ops.plan_attention_splits(batch, 1, context, nkv, nq // nkv, window, hd,
+                                                           ops.attention_wave_slots(hd))
     if window is None:
         assert splits * split_len >= context and splits > 1  # the keys are split over many waves, then merged
     bucket = ModelRunner.context_bucket(context + 1)
