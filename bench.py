@@ -379,6 +379,8 @@ def main() -> int:
     weight_bytes, layer_flops_per_token, head_flops_per_row = model_numbers(cfg, elem)
 
     def decode_point(batch, steps, warmup):
+        if batch > 64 and short == "bf16":
+            runner.warm_up([batch])  # beyond 64 rows the products are the library's: tuned for this many rows
         sec = time_decode(parts, batch, args.context, steps, warmup, args.sampled)
         log(f"decode batch {batch}{' (sampled)' if args.sampled else ''}: {sec * 1e3:.3f} ms/step, {batch / sec:.1f} tok/s")
         return sec

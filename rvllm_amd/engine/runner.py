@@ -80,12 +80,23 @@ class ModelRunner:
         self._graphs: collections.OrderedDict[tuple[int, int], tuple] = collections.OrderedDict()
         self._graph_pool = None
         self.graph_replays = 0
+        # Whether steps whose products go to the library may come from graphs: only for models that keep nothing
+        # but keys and values between steps (replaying such a step writes the same keys and values again, so the
+        # check below may replay it; a state that a mixer moves on would be moved on with every replay), and
+        # until a recording fails its check.
+        self._library_steps_from_graphs = all(need is None or isinstance(need, KVNeed) for need in needs)
         _freeze_what_exists_once()
 
     # ---- decode steps from captured graphs -------------------------------
     GRAPH_CONTEXT_BUCKET = 1024
-    GRAPH_MAX_REQUESTS = ops.SKINNY_MAX_ROWS  # beyond this the products go to the library, which stays out of graphs
     GRAPH_MAX_KEPT = 128     # shapes whose graphs are kept; the one unused for longest goes first
+    # Steps of more requests than the few-row product takes hand their products to the library.  A recording of
+    # library calls is trusted only after it has shown itself right: it is replayed this many times against the
+    # logits of the same step run kernel by kernel (nodes that a library records have given wrong results on
+    # replays after the first on this hardware), and if one replay differs no step with library products is
+    # taken from a graph again.
+    GRAPH_LIBRARY_CHECKS = 3
+    GRAPH_LIBRARY_TOLERANCE = 1e-3  # of the largest logit: the library may add in another order, not more
 
     def _graph_key(self, batch: StepBatch):
         """The key of the captured graph that can run this batch, or None.
@@ -102,9 +113,11 @@ class ModelRunner:
 
     def _decode_graph_key(self, num_requests: int, max_context: int):
         """The key for a step of ``num_requests`` decoded tokens, all wanted, at contexts up to ``max_context``."""
-        if not (self.config.use_graphs and self.dtype == torch.bfloat16) or num_requests > self.GRAPH_MAX_REQUESTS:
+        if not (self.config.use_graphs and self.dtype == torch.bfloat16):
             return None
         if not self.model.capturable:  # a part waits for the device or launches by its data
+            return None
+        if num_requests > ops.SKINNY_MAX_ROWS and not self._library_steps_from_graphs:
             return None
         return num_requests, self.context_bucket(max_context)
 
@@ -145,6 +158,11 @@ class ModelRunner:
                     gc.enable()
             if self._graph_pool is None:
                 self._graph_pool = graph.pool()
+            if key[0] > ops.SKINNY_MAX_ROWS and not self._recording_is_right(graph, static_logits, logits):
+                self._library_steps_from_graphs = False
+                warnings.warn("a recorded decode step with library products did not reproduce the step run kernel "
+                              "by kernel; such steps are no longer taken from graphs")
+                return logits
             self._graphs[key] = (graph, static_logits)
             while len(self._graphs) > self.GRAPH_MAX_KEPT:
                 self._graphs.popitem(last=False)
@@ -154,6 +172,18 @@ class ModelRunner:
         graph.replay()
         self.graph_replays += 1
         return static_logits
+
+    def _recording_is_right(self, graph, static_logits: torch.Tensor, logits: torch.Tensor) -> bool:
+        """Replays a fresh recording several times, with a wait for the device between the replays, and holds
+        every result against the logits of the same step run kernel by kernel."""
+        scale = float(logits.abs().max())
+        for _ in range(self.GRAPH_LIBRARY_CHECKS):
+            graph.replay()
+            torch.cuda.synchronize()
+            worst = float((static_logits - logits).abs().max())
+            if not worst <= self.GRAPH_LIBRARY_TOLERANCE * scale:  # NaN fails too
+                return False
+        return True
 
     # ---- construction --------------------------------------------------
     @classmethod

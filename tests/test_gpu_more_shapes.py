@@ -129,8 +129,9 @@ def many_requests_trace(vocab, count, seed, prompt_lengths=(3, 19), decode=6):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,count", [("A", 80), ("D", 65)])
 def test_more_decoding_requests_than_the_few_row_product_takes(model_dirs, plain_models, tmp_path, name, count, dtype):
-    """65 to 80 live requests decode together: beyond 64 rows the bf16 products go to the library and the step is
-    not taken from a graph; every request's logits still equal the plain implementation's."""
+    """65 to 80 live requests decode together: beyond 64 rows the bf16 products go to the library; such a step is
+    recorded too, and the recording replayed three times against the step run kernel by kernel before it is
+    trusted; every request's logits still equal the plain implementation's."""
     assert count > ops.SKINNY_MAX_ROWS
     if name == "D":
         folder = tiny_models.write_model(tmp_path / "D", "D")
@@ -140,7 +141,8 @@ def test_more_decoding_requests_than_the_few_row_product_takes(model_dirs, plain
     seqs, steps = many_requests_trace(cfg["vocab"], count, seed=count)
     runner = runner_for(folder, dtype, 64 * count, max_num_seqs=count)
     got = tt.collect(steps, tt.run_in_process(runner, steps), cfg["vocab"])
-    assert runner.graph_replays == 0
+    assert (runner.graph_replays >= 4) == (dtype == "bfloat16")  # the six decode steps but the first
+    assert runner._library_steps_from_graphs
     for rid in list(seqs)[:: 1 if name == "A" else 8]:  # the wide model's reference on the CPU is slow: every eighth
         ref = plain_gemma.forward(weights, cfg, seqs[rid], torch.float64)
         want = ref[len(seqs[rid]) - 7:]  # the prompt's last place and the six decoded ones
@@ -200,6 +202,23 @@ def test_a_head_size_above_256_and_17_query_heads_a_group(tmp_path, dtype, mode)
     prefix = steps[0]["entries"][0]["id"].split("-")[0]
     for rid, ids in seqs.items():
         tt.compare(got[f"{prefix}-{rid}"], plain_gemma.forward(weights, cfg, ids, torch.float64), dtype, f"G {mode} {rid}")
+
+
+def test_a_recording_that_does_not_reproduce_its_step_is_not_trusted(model_dirs):
+    """The check of a recorded step with library products, made to fail from the host: the step's logits come from
+    the run kernel by kernel, no graph is kept, and later steps of that kind are not recorded again; steps of few
+    requests still come from graphs."""
+    seqs, steps = many_requests_trace(256, 70, seed=3)
+    runner = runner_for(model_dirs["A"], "bfloat16", 64 * 70, max_num_seqs=70)
+    runner.GRAPH_LIBRARY_TOLERANCE = -1.0  # nothing is close enough
+    with pytest.warns(UserWarning, match="did not reproduce"):
+        tt.collect(steps, tt.run_in_process(runner, steps), 256)
+    assert runner.graph_replays == 0 and not runner._library_steps_from_graphs and not runner._graphs
+    runner.add_request("few")
+    runner.step([("few", [1, 2, 3], [])])
+    for token in (4, 5, 6):
+        runner.step([("few", [token], [0])])
+    assert runner.graph_replays >= 2
 
 
 # ---- a folder in several shards ------------------------------------------------------------------------------
