@@ -373,7 +373,8 @@ def main() -> int:
     t0 = time.time()
     runner = ModelRunner.from_random(cfg, 0, engine_cfg)
     torch.cuda.synchronize()
-    log(f"model ready in {time.time() - t0:.1f} s; cache {runner.storage.bytes / 2**30:.1f} GiB")
+    log(f"model ready in {time.time() - t0:.1f} s; weights {runner.weight_bytes / 2**30:.1f} GiB, "
+        f"cache {runner.storage.bytes / 2**30:.1f} GiB")
     parts = (torch, runner, Sampler(cfg.vocab_size), SamplingParams, SplitMix64)
 
     weight_bytes, layer_flops_per_token, head_flops_per_row = model_numbers(cfg, elem)

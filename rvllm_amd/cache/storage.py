@@ -23,13 +23,49 @@ from ..parts.base import KVCacheView, KVNeed, StateNeed, StateView
 from .manager import CacheManager
 
 
+class CacheTooLarge(MemoryError):
+    pass
+
+
+def bytes_needed(manager: CacheManager, dtype: torch.dtype) -> int:
+    """What ``CacheStorage`` allocates for these books."""
+    elem = torch.empty((), dtype=dtype).element_size()
+    total = 0
+    for i, need in enumerate(manager.needs):
+        if isinstance(need, KVNeed):
+            g = manager.groups[manager.layer_group[i]]
+            total += 2 * g.pool.num_pages * need.num_kv_heads * g.page_size * need.head_dim * elem
+        elif isinstance(need, StateNeed):
+            count = 1
+            for n in need.shape:
+                count *= int(n)
+            total += manager.max_requests * count * torch.empty((), dtype=need.dtype).element_size()
+    return total
+
+
 class CacheStorage:
-    def __init__(self, manager: CacheManager, device, dtype: torch.dtype):
+    def __init__(self, manager: CacheManager, device, dtype: torch.dtype, held_by_weights: Optional[int] = None):
+        """``held_by_weights``: the bytes the model's weights take on the device (for the message, should the cache
+        not fit beside them)."""
         self.manager = manager
         self.device = torch.device(device)
         self.dtype = dtype
         self.views: list = []
         self.bytes = 0
+        if self.device.type == "cuda":
+            # Said before the first allocation, with the numbers: the allocator's own complaint comes at some layer
+            # in the middle and names neither the cache's size nor what the weights hold.
+            need_bytes = bytes_needed(manager, dtype)
+            free, total = torch.cuda.mem_get_info(self.device)
+            free += torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
+            if need_bytes > free:
+                weights = "" if held_by_weights is None else (
+                    f"; the weights hold {held_by_weights / 2**30:.1f} GiB (bf16 matrices lie there twice while "
+                    f"tiled_weights is on: row by row for the library's products, in tiles for decode steps)")
+                raise CacheTooLarge(
+                    f"the cache for {manager.max_requests} requests needs {need_bytes / 2**30:.1f} GiB, "
+                    f"{free / 2**30:.1f} GiB of {total / 2**30:.1f} GiB are free{weights}; lower max_cache_tokens, "
+                    f"max_num_seqs or max_model_len")
         for i, need in enumerate(manager.needs):
             if isinstance(need, KVNeed):
                 g = manager.groups[manager.layer_group[i]]

@@ -72,7 +72,8 @@ class ModelRunner:
                     per_request = window_pages_bound(need.window, ps, cfg.max_num_batched_tokens)
                     num_pages[name] = min(full_pages, cfg.max_num_seqs * per_request)
         self.cache = CacheManager(needs, ps, num_pages, cfg.max_num_seqs)
-        self.storage = CacheStorage(self.cache, self.device, self.dtype)
+        self.weight_bytes = model.weight_bytes()
+        self.storage = CacheStorage(self.cache, self.device, self.dtype, held_by_weights=self.weight_bytes)
         width = -(-cfg.max_model_len // ps)
         self.builder = BatchBuilder(self.device, cfg.max_num_batched_tokens, cfg.max_num_seqs,
                                     {name: width for name in self.cache.groups})
@@ -156,13 +157,14 @@ class ModelRunner:
             finally:
                 if collecting:
                     gc.enable()
-            if self._graph_pool is None:
-                self._graph_pool = graph.pool()
             if key[0] > ops.SKINNY_MAX_ROWS and not self._recording_is_right(graph, static_logits, logits):
+                # (the graph goes, and with it its memory; it has not lent its pool to the others yet)
                 self._library_steps_from_graphs = False
                 warnings.warn("a recorded decode step with library products did not reproduce the step run kernel "
                               "by kernel; such steps are no longer taken from graphs")
                 return logits
+            if self._graph_pool is None:
+                self._graph_pool = graph.pool()
             self._graphs[key] = (graph, static_logits)
             while len(self._graphs) > self.GRAPH_MAX_KEPT:
                 self._graphs.popitem(last=False)

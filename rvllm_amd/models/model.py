@@ -65,6 +65,29 @@ class DecoderModel:
         self.final_norm.bind(tensors, self.spec.prefix, self.device, dtype)
         self.head.bind(tensors, self.spec.prefix, self.device, dtype)
 
+    def weight_bytes(self) -> int:
+        """Bytes the bound weights take on the device, every allocation counted once (a tied head shares the
+        embedding's table; a matrix in tiles counts with the rows kept beside it)."""
+        from ..kernels.ops import TiledWeight
+
+        seen: dict[int, int] = {}
+
+        def count(value):
+            if isinstance(value, TiledWeight):
+                count(value.tiles)
+                count(value.rows)
+            elif isinstance(value, torch.Tensor) and value.device.type != "cpu":
+                storage = value.untyped_storage()
+                seen[storage.data_ptr()] = storage.nbytes()
+            elif isinstance(value, (list, tuple)):
+                for item in value:
+                    count(item)
+
+        for part in self.all_parts():
+            for value in vars(part).values():
+                count(value)
+        return sum(seen.values())
+
     @property
     def capturable(self) -> bool:
         """Whether a step of this model may be recorded into a HIP graph: only if every part may."""

@@ -288,6 +288,25 @@ def test_pages_change_hands_in_a_mixed_trace(model_dirs, plain_models, dtype):
         assert shared, f"no page of group {name} was held by two requests"
 
 
+# ---- memory ------------------------------------------------------------------------------------------------
+def test_weights_are_counted_and_a_cache_that_does_not_fit_is_refused_with_the_numbers(model_dirs, monkeypatch):
+    from rvllm_amd.cache.storage import CacheTooLarge
+
+    tiled = runner_for(model_dirs["B"], "bfloat16", 256)
+    rows = runner_for(model_dirs["B"], "bfloat16", 256, tiled_weights=False)
+    params = sum(t.numel() for t in plain_gemma.load_weights(model_dirs["B"]).values())
+    assert rows.weight_bytes == 2 * params  # bf16, the tied head's table once
+    # in tiles every matrix lies there a second time, its rows and columns filled up to whole tiles
+    assert 1.9 * rows.weight_bytes < tiled.weight_bytes < 2.6 * rows.weight_bytes
+    # a device with 64 MiB free (said by the host: nothing is filled up for this)
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (64 << 20, 288 << 30))
+    monkeypatch.setattr(torch.cuda, "memory_reserved", lambda device=None: torch.cuda.memory_allocated(device))
+    with pytest.raises(CacheTooLarge, match=r"needs \d+\.\d GiB, 0\.1 GiB of 288\.0 GiB are free; the weights hold"):
+        ModelRunner.from_model_dir(model_dirs["B"], EngineConfig(dtype="bfloat16", max_model_len=2048, max_num_seqs=64,
+                                                                 max_cache_tokens=600_000))
+    runner_for(model_dirs["B"], "bfloat16", 256)  # what fits is built as ever
+
+
 # ---- logits of replayed steps ----------------------------------------------------------------------------
 def test_logits_of_a_replayed_step_live_until_the_next_step_of_its_shape(model_dirs):
     """A decode step replayed from a graph returns the graph's own output buffer: the next step of the same shape
