@@ -21,7 +21,7 @@ a token may see) over its time.  ``prefill.frac`` prices the prompt's flops
 against 2.5 PFLOP/s (dense bf16 MFMA).  Beside the vendor's peaks stand
 measured ones (``measured_peak``): what a kernel that only reads gets from the
 memory (the engine's own probe kernel over 4 GiB), and what the library's bf16
-product of 8192 x 8192 x 8192 reaches (hipBLASLt through torch.matmul).
+product of 8192 x 8192 x 8192 reaches (hipBLASLt, called as the engine calls it).
 
 The timed decode steps end at the named context: the caches are filled so that
 the last timed step sees exactly ``--context`` tokens, and every step runs
@@ -213,7 +213,7 @@ def measure_peaks(torch, device, short: str) -> dict:
         best = None
         for i in range(6):
             start.record()
-            torch.matmul(a, b.t(), out=c)
+            ops.library_gemm(a, b, c)
             stop.record()
             stop.synchronize()
             ms = start.elapsed_time(stop)

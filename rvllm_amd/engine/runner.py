@@ -222,20 +222,12 @@ class ModelRunner:
         """Runs a throw-away prompt portion of each given length so that what
         is chosen or built at first use is ready before requests arrive.  For
         bf16 the library's matrix products (portions of more than 64 tokens)
-        are tuned meanwhile: torch's TunableOp times the library's candidate
-        kernels for each shape once and keeps the fastest; afterwards tuning
-        is switched off again, so a shape met later costs no pause."""
-        import torch.cuda.tunable as tunable
-
+        are tuned meanwhile: every algorithm the library has for a shape is
+        timed once and the fastest kept (``ops.set_library_tuning``);
+        afterwards tuning is switched off again, so a shape met later costs
+        no pause and runs on the library's first suggestion."""
         tune = self.dtype == torch.bfloat16 and any(n > ops.SKINNY_MAX_ROWS for n in portion_lengths)
-        if tune:
-            tunable.enable(True)
-            tunable.tuning_enable(True)
-            tunable.set_max_tuning_duration(150)
-            tunable.set_max_tuning_iterations(30)
-            # the results are kept beside the system's temporary files, not in the working folder
-            import tempfile
-            tunable.set_filename(os.path.join(tempfile.gettempdir(), f"rvllm_amd_tunable_{os.getuid()}.csv"))
+        ops.set_library_tuning(tune)
         try:
             for n in portion_lengths:
                 n = min(int(n), self.config.max_num_batched_tokens, self.config.max_model_len)
@@ -248,8 +240,7 @@ class ModelRunner:
                     self.release("__warm_up__")
             torch.cuda.synchronize(self.device)
         finally:
-            if tune:
-                tunable.tuning_enable(False)
+            ops.set_library_tuning(False)
 
     # ---- requests ----------------------------------------------------
     def add_request(self, request: Hashable) -> None:

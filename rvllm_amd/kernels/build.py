@@ -39,6 +39,8 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument",
     "-Wno-inline-asm",  # the copies into LDS name the register m0, which the compiler calls reserved
 ]
+# The products of many rows go to hipBLASLt (csrc/library_gemm.hip).
+LINK_FLAGS = ["-lhipblaslt"]
 LIB_STEM = "librvllm_amd"
 
 
@@ -55,7 +57,7 @@ def source_hash() -> str:
     for path in _sources() + _headers():
         h.update(path.name.encode())
         h.update(path.read_bytes())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HIPCC_FLAGS + LINK_FLAGS).encode())
     return h.hexdigest()[:12]
 
 
@@ -143,7 +145,7 @@ def build(force: bool = True, jobs: int | None = None) -> Path:
                 done += 1
                 _say(f"  [{done}/{len(srcs)}] {src.name} ({secs:.1f} s)")
         tmp_lib = Path(tmp) / name
-        link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp_lib), *map(str, objs)]
+        link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp_lib), *map(str, objs), *LINK_FLAGS]
         proc = subprocess.run(link, capture_output=True, text=True)
         if proc.returncode != 0:
             raise RuntimeError(f"link failed:\n{proc.stderr[-4000:]}")

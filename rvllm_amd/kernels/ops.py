@@ -873,6 +873,69 @@ def gemm_bf16(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,
 
 SKINNY_MAX_ROWS = 64
 
+# ---- products of many rows: the library's --------------------------------------------------------------------
+LIBRARY_WORKSPACE_BYTES = 64 << 20
+_library_workspaces: dict = {}
+_library_tuning = False
+
+
+def library_workspace(device) -> torch.Tensor:
+    """The device memory that the library's algorithms may use, one allocation a device, made at first use."""
+    index = torch.device(device).index or 0
+    ws = _library_workspaces.get(index)
+    if ws is None:
+        ws = _library_workspaces[index] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    return ws
+
+
+def set_library_tuning(on: bool) -> None:
+    """While on, ``library_gemm`` first times the library's algorithms for every shape it has not tuned yet and
+    keeps the fastest (a second or so a shape, with a wait for the device): for warm-up runs, never inside a
+    recording."""
+    global _library_tuning
+    _library_tuning = bool(on)
+
+
+def _library_args(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
+    _need(x.is_cuda and w.is_cuda and out.is_cuda, "library product: arguments must live on the GPU")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
+          "library product: bfloat16 only")
+    _need(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "library product: matrices expected")
+    m, k = x.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n), "library product: shapes do not fit")
+    _need(x.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "library product: rows must be contiguous")
+    ws = library_workspace(x.device)
+    return (_ptr(x), _ptr(w), _ptr(out), _c_int(m), _c_int(n), _c_int(k), _c_ll(x.stride(0) if m > 1 else k),
+            _c_ll(w.stride(0) if n > 1 else k), _c_ll(out.stride(0) if m > 1 else n), _ptr(ws), _c_ll(ws.numel()))
+
+
+def library_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optional[torch.Tensor]:
+    """out[M, N] = x[M, K] @ w[N, K]^T in bf16 with 32-bit sums, by hipBLASLt (``csrc/library_gemm.hip``): the
+    product of more rows than the few-row kernel takes.  A shape keeps its plan; see ``set_library_tuning``.
+    None, with nothing done, for a shape that the library has no algorithm for."""
+    args = _library_args(x, w, out)
+    lib = library()
+    if _library_tuning:
+        _check(min(0, lib.rv_lt_tune(_stream(), *args, _c_int(LIBRARY_TUNE_BUDGET_MS))))
+    status = lib.rv_lt_gemm(_stream(), *args)
+    if status == 2:  # the library has no algorithm for this shape: nothing ran
+        return None
+    _check(status)
+    return out
+
+
+LIBRARY_TUNE_BUDGET_MS = 3000
+
+
+def library_plan_info(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tuple[int, int, float]:
+    """(1 tuned / 0 the library's first suggestion / -1 never seen, the algorithm's index, the time it was tuned
+    to in microseconds) for the shape of this product."""
+    args = _library_args(x, w, out)
+    index, us = ctypes.c_int(-1), ctypes.c_float(0.0)
+    state = library().rv_lt_plan_info(*args[3:9], ctypes.byref(index), ctypes.byref(us))
+    return state, index.value, us.value
+
 
 def probe_read(data: torch.Tensor, blocks: int = 2048) -> torch.Tensor:
     """Reads ``data`` once with a kernel that does nothing else (a measurement of the memory's read rate);

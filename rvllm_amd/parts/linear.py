@@ -1,8 +1,9 @@
 """Matrix products of the parts: out = x @ w^T.
 
 The 32-bit path uses the hand-written kernel with 32-bit multiply-adds only.
-The bf16 path hands plain products to the library through torch (hipBLASLt /
-rocBLAS), as the reference hands its products to cuBLASLt
+The bf16 path hands plain products of many rows to the library (hipBLASLt,
+called from the kernel library itself: ``csrc/library_gemm.hip``), as the
+reference hands its products to cuBLASLt
 (v3/crates/rvllm-cutlass/src/cublaslt.rs:277); products with few rows, and
 products with 32-bit output from bf16 inputs (the logits), run on the
 hand-written kernels.
@@ -74,7 +75,7 @@ def linear(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,
             raise ops.KernelError(f"linear: unsupported weight dtype {w.dtype}")
         return ops.gemm_plain(x, w, out)
     if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-        if out.dtype == torch.bfloat16:
-            return torch.matmul(x, w.t(), out=out)
+        if out.dtype == torch.bfloat16 and ops.library_gemm(x, w, out) is not None:
+            return out
         return ops.gemm_plain(x, w, out)
     raise ops.KernelError(f"linear: unsupported dtypes x={x.dtype} w={w.dtype}")

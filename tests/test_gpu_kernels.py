@@ -303,6 +303,62 @@ def test_gemm_skinny_reads_strided_rows_and_refuses_what_it_cannot():
                          torch.empty((2, 4), dtype=torch.float32, device=DEV)) is None  # K is no multiple of 8
 
 
+LIBRARY_SHAPES = [(65, 96, 64), (128, 2048 + 64, 3840), (300, 1000, 2560), (2048, 264, 1152), (77, 112, 72),
+                  (200, 333, 40)]
+
+
+@pytest.mark.parametrize("m,n,k", LIBRARY_SHAPES)
+def test_the_librarys_product_against_64_bit(m, n, k):
+    """The product of many rows goes to hipBLASLt from the kernel library itself; a shape that the library has no
+    algorithm for comes back as None with nothing written, and ``linear`` takes the plain kernel for it."""
+    from rvllm_amd.parts.linear import linear
+
+    g = torch.Generator().manual_seed(m + n + k)
+    x = dev(torch.randn(m, k, generator=g).bfloat16())
+    w = dev((torch.randn(n, k, generator=g) * k ** -0.5).bfloat16())
+    want = x.cpu().double() @ w.cpu().double().T
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    got = ops.library_gemm(x, w, out)
+    if got is None:
+        assert bool(torch.isnan(out).all())
+    else:
+        assert got is out
+        assert torch.allclose(out.cpu().double(), want, atol=2e-2, rtol=1e-2)
+    assert torch.allclose(linear(x, w).cpu().double(), want, atol=2e-2, rtol=1e-2)
+    # rows that lie apart, in x and in out (a slice of a wider buffer, as the fused projections' outputs are)
+    wide_x = dev(torch.randn(m, k + 24, generator=g).bfloat16())
+    wide_out = torch.full((m, n + 40), 7.0, dtype=torch.bfloat16, device=DEV)
+    xs, outs = wide_x[:, 8:8 + k], wide_out[:, 16:16 + n]
+    linear(xs, w, out=outs)
+    assert torch.allclose(outs.cpu().double(), xs.cpu().double() @ w.cpu().double().T, atol=2e-2, rtol=1e-2)
+    assert bool((wide_out[:, :16] == 7.0).all()) and bool((wide_out[:, 16 + n:] == 7.0).all())
+
+
+def test_the_librarys_product_tuned_gives_the_same_and_keeps_its_plan():
+    g = torch.Generator().manual_seed(5)
+    m, n, k = 160, 512 + 32, 640
+    x = dev(torch.randn(m, k, generator=g).bfloat16())
+    w = dev((torch.randn(n, k, generator=g) * k ** -0.5).bfloat16())
+    want = x.cpu().double() @ w.cpu().double().T
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    assert ops.library_gemm(x, w, out) is out
+    assert ops.library_plan_info(x, w, out)[0] == 0  # the library's first suggestion
+    first = out.clone()
+    ops.set_library_tuning(True)
+    try:
+        assert ops.library_gemm(x, w, out) is out
+    finally:
+        ops.set_library_tuning(False)
+    state, index, us = ops.library_plan_info(x, w, out)
+    assert state == 1 and index >= 0 and 0.0 < us < 1000.0
+    assert torch.allclose(out.cpu().double(), want, atol=2e-2, rtol=1e-2)
+    assert torch.allclose(out.float(), first.float(), atol=2e-2, rtol=1e-2)
+    out.fill_(float("nan"))
+    ops.library_gemm(x, w, out)  # the kept plan, with tuning off
+    assert ops.library_plan_info(x, w, out) == (state, index, us)
+    assert torch.allclose(out.cpu().double(), want, atol=2e-2, rtol=1e-2)
+
+
 def paged_setup(T_total, nkv, hd, page_size, dtype, seed, scramble=True):
     """A cache whose pages are handed out in a scrambled order."""
     g = torch.Generator().manual_seed(seed)
