@@ -17,6 +17,7 @@
 #include <hipblaslt/hipblaslt.h>
 
 #include <algorithm>
+#include <cstdio>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -257,4 +258,83 @@ extern "C" int rv_lt_plan_info(int M, int N, int K, long long ldx, long long ldw
   if (algo_index) *algo_index = it->second.algo_index;
   if (tuned_us) *tuned_us = it->second.tuned_us;
   return it->second.tuned ? 1 : 0;
+}
+
+// The library's version (its number, as hipblasLtGetVersion gives it): an algorithm's index means something only
+// to the version that gave it.  -1 on an error.
+extern "C" int rv_lt_version(void) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return -1;
+  std::lock_guard<std::mutex> guard(g_lock);
+  hipblasLtHandle_t handle;
+  if (handle_for(dev, &handle)) return -1;
+  int version = -1;
+  if (hipblasLtGetVersion(handle, &version) != HIPBLAS_STATUS_SUCCESS) return -1;
+  return version;
+}
+
+// What kind of device the current one is, for the file of plans: its architecture's name and its number of compute
+// units, as text in `out` (at most `room` bytes with the final 0).  0 or -1.
+extern "C" int rv_lt_device_kind(char* out, int room) {
+  int dev = 0;
+  hipDeviceProp_t prop;
+  RV_CHECK(out && room > 0, "library product: no room for the device's kind");
+  RV_CHECK(hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess,
+           "library product: the current device's properties cannot be read");
+  snprintf(out, (size_t)room, "%s/%d", prop.gcnArchName, prop.multiProcessorCount);
+  return 0;
+}
+
+// The `i`-th tuned shape of the current device, in no particular order: 1 and the shape, its algorithm's index and
+// its time; 0 when there are fewer.
+extern "C" int rv_lt_tuned_plan(int i, int* M, int* N, int* K, long long* ldx, long long* ldw, long long* ldc,
+                                int* algo_index, float* tuned_us) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  std::lock_guard<std::mutex> guard(g_lock);
+  for (const auto& kv : g_plans) {
+    if (kv.first.dev != dev || !kv.second.tuned || kv.second.none) continue;
+    if (i-- > 0) continue;
+    *M = kv.first.M, *N = kv.first.N, *K = kv.first.K;
+    *ldx = kv.first.ldx, *ldw = kv.first.ldw, *ldc = kv.first.ldc;
+    *algo_index = kv.second.algo_index;
+    *tuned_us = kv.second.tuned_us;
+    return 1;
+  }
+  return 0;
+}
+
+// Takes an algorithm that an earlier run of the same library tuned this shape to, by its index, instead of tuning
+// again: 0 if it is taken (the shape then counts as tuned), RV_LT_NO_ALGORITHM if the library does not know the index
+// or the algorithm does not take the shape (nothing changes: the shape runs on the first suggestion and can be
+// tuned), -1 on an error.
+extern "C" int rv_lt_take_plan(int M, int N, int K, long long ldx, long long ldw, long long ldc, int algo_index,
+                               float tuned_us, long long workspace_bytes) {
+  RV_CHECK(M > 0 && N > 0 && K > 0 && ldx >= K && ldw >= K && ldc >= N && algo_index >= 0,
+           "library product: bad plan M=%d N=%d K=%d index=%d", M, N, K, algo_index);
+  int dev = 0;
+  RV_CHECK(hipGetDevice(&dev) == hipSuccess, "library product: no current device");
+  std::lock_guard<std::mutex> guard(g_lock);
+  hipblasLtHandle_t handle;
+  if (handle_for(dev, &handle)) return -1;
+  LtPlan* plan;
+  if (plan_for(handle, LtShape{dev, M, N, K, ldx, ldw, ldc}, (size_t)workspace_bytes, &plan)) return -1;
+  if (plan->tuned) return 0;
+  if (plan->none) return RV_LT_NO_ALGORITHM;
+  std::vector<int> wanted{algo_index};
+  std::vector<hipblasLtMatmulHeuristicResult_t> found;
+  if (hipblaslt_ext::getAlgosFromIndex(handle, wanted, found) != HIPBLAS_STATUS_SUCCESS || found.empty())
+    return RV_LT_NO_ALGORITHM;
+  const float one = 1.f, zero = 0.f;
+  size_t room = 0;
+  if (hipblaslt_ext::matmulIsAlgoSupported(handle, plan->desc, &one, plan->a, plan->b, &zero, plan->d, plan->d,
+                                           found[0].algo, room) != HIPBLAS_STATUS_SUCCESS ||
+      room > (size_t)workspace_bytes)
+    return RV_LT_NO_ALGORITHM;
+  plan->algo = found[0].algo;
+  plan->workspace = room;
+  plan->algo_index = hipblaslt_ext::getIndexFromAlgo(plan->algo);
+  plan->tuned = true;
+  plan->tuned_us = tuned_us;
+  return 0;
 }

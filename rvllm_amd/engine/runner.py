@@ -225,8 +225,13 @@ class ModelRunner:
         are tuned meanwhile: every algorithm the library has for a shape is
         timed once and the fastest kept (``ops.set_library_tuning``);
         afterwards tuning is switched off again, so a shape met later costs
-        no pause and runs on the library's first suggestion."""
+        no pause and runs on the library's first suggestion.  If the
+        environment names a file (``ops.LIBRARY_PLANS_ENV``), the plans in it
+        are taken first, and what is tuned now is written there."""
         tune = self.dtype == torch.bfloat16 and any(n > ops.SKINNY_MAX_ROWS for n in portion_lengths)
+        plans_file = os.environ.get(ops.LIBRARY_PLANS_ENV) if tune else None
+        if plans_file:
+            ops.library_plans_load(plans_file, self.device)
         ops.set_library_tuning(tune)
         try:
             for n in portion_lengths:
@@ -241,6 +246,8 @@ class ModelRunner:
             torch.cuda.synchronize(self.device)
         finally:
             ops.set_library_tuning(False)
+        if plans_file:
+            ops.library_plans_save(plans_file, self.device)
 
     # ---- requests ----------------------------------------------------
     def add_request(self, request: Hashable) -> None:

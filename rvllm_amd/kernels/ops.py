@@ -926,6 +926,73 @@ def library_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optiona
 
 
 LIBRARY_TUNE_BUDGET_MS = 3000
+# The environment variable that names a file of tuned plans: ``ModelRunner.warm_up`` reads it before it tunes and
+# writes it afterwards, so that a later start finds its shapes tuned.
+LIBRARY_PLANS_ENV = "RVLLM_AMD_LIBRARY_PLANS"
+
+
+def _library_plans_key(device) -> dict:
+    """What a file of plans holds for: an algorithm's index means something only to one version of the library on
+    one kind of device."""
+    kind = ctypes.create_string_buffer(128)
+    with torch.cuda.device(device):
+        _check(library().rv_lt_device_kind(kind, _c_int(len(kind))))
+        return {"device": kind.value.decode(), "hipblaslt": int(library().rv_lt_version())}
+
+
+def library_plans_save(path: str, device) -> int:
+    """Writes the tuned shapes of ``device`` (shape, strides, the algorithm's index, its time) to ``path`` as JSON,
+    over what the file held; the number of shapes written."""
+    import json
+    import os
+
+    lib = library()
+    plans = []
+    with torch.cuda.device(device):
+        while True:
+            m, n, k, index = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+            ldx, ldw, ldc = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_longlong()
+            us = ctypes.c_float()
+            if not lib.rv_lt_tuned_plan(_c_int(len(plans)), ctypes.byref(m), ctypes.byref(n), ctypes.byref(k),
+                                        ctypes.byref(ldx), ctypes.byref(ldw), ctypes.byref(ldc), ctypes.byref(index),
+                                        ctypes.byref(us)):
+                break
+            plans.append([m.value, n.value, k.value, ldx.value, ldw.value, ldc.value, index.value, round(us.value, 2)])
+        doc = dict(_library_plans_key(device), plans=sorted(plans))
+    tmp = f"{path}.{os.getpid()}.tmp"
+    with open(tmp, "w") as f:
+        json.dump(doc, f, indent=0)
+    os.replace(tmp, path)
+    return len(plans)
+
+
+def library_plans_load(path: str, device) -> int:
+    """Takes the plans of a file written by ``library_plans_save``: the number of shapes that now count as tuned.
+    A file that is missing, unreadable, or of another device or version of the library gives 0 and changes nothing;
+    so does a plan that the library does not take."""
+    import json
+
+    try:
+        with open(path) as f:
+            doc = json.load(f)
+        plans = [(int(m), int(n), int(k), int(ldx), int(ldw), int(ldc), int(index), float(us))
+                 for m, n, k, ldx, ldw, ldc, index, us in doc["plans"]]
+    except (OSError, ValueError, KeyError, TypeError):
+        return 0
+    lib = library()
+    taken = 0
+    with torch.cuda.device(device):
+        if {key: doc.get(key) for key in ("device", "hipblaslt")} != _library_plans_key(device):
+            return 0
+        room = library_workspace(torch.device(device)).numel()
+        for m, n, k, ldx, ldw, ldc, index, us in plans:
+            status = lib.rv_lt_take_plan(_c_int(m), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(ldc),
+                                         _c_int(index), _c_float(us), _c_ll(room))
+            if status == 0:
+                taken += 1
+            elif status != 2:
+                _check(status)
+    return taken
 
 
 def library_plan_info(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tuple[int, int, float]:

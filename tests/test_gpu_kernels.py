@@ -359,6 +359,57 @@ def test_the_librarys_product_tuned_gives_the_same_and_keeps_its_plan():
     assert torch.allclose(out.cpu().double(), want, atol=2e-2, rtol=1e-2)
 
 
+def test_the_librarys_tuned_plans_go_to_a_file_and_come_back(tmp_path):
+    """What tuning found is written as JSON and taken again by index: a plan for a shape this process has not
+    seen makes the shape count as tuned (or is refused, if the algorithm does not take the shape) and the product
+    is right either way; a file of another version of the library, a broken one and a missing one change nothing."""
+    import json
+
+    g = torch.Generator().manual_seed(6)
+    m, n, k = 176, 384 + 32, 704
+    x = dev(torch.randn(m, k, generator=g).bfloat16())
+    w = dev((torch.randn(n, k, generator=g) * k ** -0.5).bfloat16())
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    ops.set_library_tuning(True)
+    try:
+        ops.library_gemm(x, w, out)
+    finally:
+        ops.set_library_tuning(False)
+    state, index, us = ops.library_plan_info(x, w, out)
+    assert state == 1
+    path = tmp_path / "plans.json"
+    assert ops.library_plans_save(str(path), DEV) >= 1
+    doc = json.loads(path.read_text())
+    assert [m, n, k, k, k, n, index] in [p[:7] for p in doc["plans"]]
+    assert ops.library_plans_load(str(path), DEV) == len(doc["plans"])  # all known already: they stay as they are
+
+    m2 = m + 16  # a shape nobody has tuned here, under the first one's algorithm
+    x2 = dev(torch.randn(m2, k, generator=g).bfloat16())
+    out2 = torch.empty((m2, n), dtype=torch.bfloat16, device=DEV)
+    assert ops.library_plan_info(x2, w, out2)[0] == -1
+    other = tmp_path / "other.json"
+    other.write_text(json.dumps(dict(doc, plans=[[m2, n, k, k, k, n, index, 12.5]])))
+    taken = ops.library_plans_load(str(other), DEV)
+    assert taken in (0, 1)
+    assert ops.library_plan_info(x2, w, out2)[:2] == ((1, index) if taken else (0, ops.library_plan_info(x2, w, out2)[1]))
+    assert ops.library_gemm(x2, w, out2) is out2
+    assert torch.allclose(out2.cpu().double(), x2.cpu().double() @ w.cpu().double().T, atol=2e-2, rtol=1e-2)
+
+    m3 = m + 32
+    x3 = dev(torch.randn(m3, k, generator=g).bfloat16())
+    out3 = torch.empty((m3, n), dtype=torch.bfloat16, device=DEV)
+    other.write_text(json.dumps(dict(doc, hipblaslt=doc["hipblaslt"] + 1, plans=[[m3, n, k, k, k, n, index, 12.5]])))
+    assert ops.library_plans_load(str(other), DEV) == 0
+    other.write_text(json.dumps(dict(doc, plans=[[m3, n, k, k, k, n, 1 << 30, 12.5]])))  # no such algorithm
+    assert ops.library_plans_load(str(other), DEV) == 0
+    other.write_text("{ not json")
+    assert ops.library_plans_load(str(other), DEV) == 0
+    assert ops.library_plans_load(str(tmp_path / "missing.json"), DEV) == 0
+    assert ops.library_plan_info(x3, w, out3)[0] in (-1, 0)
+    assert ops.library_gemm(x3, w, out3) is out3
+    assert torch.allclose(out3.cpu().double(), x3.cpu().double() @ w.cpu().double().T, atol=2e-2, rtol=1e-2)
+
+
 def paged_setup(T_total, nkv, hd, page_size, dtype, seed, scramble=True):
     """A cache whose pages are handed out in a scrambled order."""
     g = torch.Generator().manual_seed(seed)
