@@ -3,9 +3,10 @@
 Every layer with a key/value need gets one allocation, keys then values (as
 in v3/crates/rvllm-mem/src/kv_layout.rs:1-46).  Inside it keys are
 ``[num_pages, kv_heads, page_size, head_dim]`` and values are transposed
-inside the page, ``[num_pages, kv_heads, head_dim, page_size]``: what one
-key/value head holds on a page is one contiguous block, and the matrix-core
-attention kernel reads both operands in the order it sums them.  Every layer
+inside groups of 16 slots, ``[num_pages, kv_heads, page_size / 16, head_dim,
+16]``: what one key/value head holds on a page is one contiguous block, and
+the matrix-core attention kernel reads both operands in the order it sums
+them, 16 keys at a time from one run of memory whatever the page size.  Every layer
 with a fixed-size state gets ``[max_requests, *shape]``.  Nothing is cleared when pages change
 hands: a position that a token may not see is never read, so what an earlier
 request left behind is unreachable (the reference relies on the same for its
@@ -18,6 +19,8 @@ from __future__ import annotations
 from typing import Optional
 
 import torch
+
+VALUE_GROUP = 16  # slots whose values of one dimension lie side by side (csrc/kv_layout.h)
 
 from ..parts.base import KVCacheView, KVNeed, StateNeed, StateView
 from .manager import CacheManager
@@ -73,7 +76,11 @@ class CacheStorage:
                                  device=self.device)
                 self.bytes += kv.numel() * kv.element_size()
                 keys = kv[0].view(g.pool.num_pages, need.num_kv_heads, g.page_size, need.head_dim)
-                values = kv[1].view(g.pool.num_pages, need.num_kv_heads, need.head_dim, g.page_size)
+                if g.page_size % VALUE_GROUP:
+                    raise ValueError(f"page_size {g.page_size} must be a multiple of {VALUE_GROUP}: the values are "
+                                     f"transposed by groups of that many slots")
+                values = kv[1].view(g.pool.num_pages, need.num_kv_heads, g.page_size // VALUE_GROUP, need.head_dim,
+                                    VALUE_GROUP)
                 self.views.append(KVCacheView(keys, values, g.name, g.page_size))
             elif isinstance(need, StateNeed):
                 slots = torch.zeros((manager.max_requests, *need.shape), dtype=need.dtype, device=self.device)

@@ -112,6 +112,7 @@ extern "C" int rv_paged_attention_generic(hipStream_t stream, const void* q, con
   RV_CHECK(num_tokens >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention: bad head counts nq=%d nkv=%d", nq, nkv);
   RV_CHECK(hd > 0 && hd <= ATT_MAX_HD, "attention: head_dim %d must be in 1..%d", hd, ATT_MAX_HD);
   RV_CHECK(page_size > 0 && num_pages > 0 && table_width > 0, "attention: bad cache geometry");
+  RV_CHECK(page_size % RV_V_GROUP == 0, "attention: page_size %d must be a multiple of %d", page_size, RV_V_GROUP);
   RV_CHECK(window >= 0, "attention: window %d must be >= 0 (0 = every key)", window);
   if (num_tokens == 0) return 0;
   RV_CHECK((long long)num_tokens * nq < (1ll << 31), "attention: too many (token, head) pairs");

@@ -147,17 +147,18 @@ __device__ void v_write_page(long long unit, const ValuePages& V, const T* __res
   const int slot0 = lo - lp * page_size;
   constexpr int VEC = 16 / sizeof(T);  // elements of a 16-byte store
   const bool whole = hi - lo == page_size && page_size % VEC == 0;
+  static_assert(RV_V_GROUP % VEC == 0, "a 16-byte store stays inside a group of slots");
   for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    T* row = v_pages + rv_v_index(page, kvh, 0, d, nkv, page_size, hd);
     if (whole) {
       for (int g = 0; g < page_size; g += VEC) {
         T v[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) v[i] = src[(size_t)(g + i) * width + d];
-        *(uint4*)(row + g) = *(const uint4*)v;
+        *(uint4*)(v_pages + rv_v_index(page, kvh, g, d, nkv, page_size, hd)) = *(const uint4*)v;
       }
     } else {
-      for (int i = 0; i < hi - lo; ++i) row[slot0 + i] = src[(size_t)i * width + d];
+      for (int i = 0; i < hi - lo; ++i)
+        v_pages[rv_v_index(page, kvh, slot0 + i, d, nkv, page_size, hd)] = src[(size_t)i * width + d];
     }
   }
 }
@@ -228,14 +229,14 @@ __global__ void qk_norm_rope_kv_write_kernel(const void* __restrict__ qkv, int s
       dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
     } else {
       if (write_kv == 2) return;  // values are written a page at a time by other blocks of this launch
-      // values are stored as projected, transposed inside the page
+      // values are stored as projected, transposed inside their group of 16 slots
       T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
 #pragma unroll
       for (int j = 0; j < QKR_PAIRS; ++j) {
         const int i = lane + j * RV_WAVE;
         if (i < half) {
-          col[(size_t)i * page_size] = rv_from_float<T>(lo[j]);
-          col[(size_t)(i + half) * page_size] = rv_from_float<T>(hi[j]);
+          col[(size_t)i * RV_V_GROUP] = rv_from_float<T>(lo[j]);
+          col[(size_t)(i + half) * RV_V_GROUP] = rv_from_float<T>(hi[j]);
         }
       }
       return;
@@ -403,11 +404,11 @@ __global__ void qk_norm_rope_kv_write_vec_kernel(const void* __restrict__ qkv, i
       if (is_k) {
         dst = k_pages + rv_k_index(page, head - nq, slot, 0, nkv, page_size, hd);
       } else {
-        // values are stored as projected, transposed inside the page
+        // values are stored as projected, transposed inside their group of 16 slots
         T* col = v_pages + rv_v_index(page, head - nq - nkv, slot, 0, nkv, page_size, hd);
         if (active) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) col[(size_t)(d0 + i) * page_size] = rv_from_float<T>(x[j][i]);
+          for (int i = 0; i < 4; ++i) col[(size_t)(d0 + i) * RV_V_GROUP] = rv_from_float<T>(x[j][i]);
         }
         continue;
       }
@@ -557,6 +558,8 @@ extern "C" int rv_qk_norm_rope_kv_write(hipStream_t stream, const void* qkv, int
   RV_CHECK((q_w == nullptr) == (k_w == nullptr), "qk_norm_rope: query and key norm weights come together");
   RV_CHECK(!write_kv || (page_size > 0 && num_pages > 0 && table_width > 0 && block_table && k_pages && v_pages),
            "qk_norm_rope: cache write needs pages and a block table");
+  RV_CHECK(!write_kv || page_size % RV_V_GROUP == 0, "qk_norm_rope: page_size %d must be a multiple of %d", page_size,
+           RV_V_GROUP);
   if (num_tokens == 0) return 0;
   // write_kv 0: nothing goes to the cache; 1: keys and values, token by token; 2: keys token by token and values
   // a page at a time, by extra rows of blocks (for prompt portions; needs the step's portions and whole values,

@@ -99,14 +99,18 @@ def _i32(*tensors: torch.Tensor) -> None:
 _c_int, _c_float, _c_ll = int, ctypes.c_float, ctypes.c_longlong
 
 
+V_GROUP = 16  # slots whose values of one dimension lie side by side (RV_V_GROUP of csrc/kv_layout.h)
+
+
 def _cache_geometry(k_pages: torch.Tensor, v_pages: torch.Tensor, what: str) -> tuple[int, int, int, int]:
     """(pages, kv heads, page size, head size) of a layer's cache: keys are
     ``[pages, kv_heads, page_size, head_dim]``, values are transposed inside
-    the page, ``[pages, kv_heads, head_dim, page_size]``."""
-    _need(k_pages.dim() == 4 and v_pages.dim() == 4, f"{what}: cache pages must have four dimensions")
+    groups of 16 slots, ``[pages, kv_heads, page_size / 16, head_dim, 16]``."""
+    _need(k_pages.dim() == 4 and v_pages.dim() == 5, f"{what}: key pages must have four dimensions, value pages five")
     num_pages, nkv, page_size, hd = k_pages.shape
-    _need(tuple(v_pages.shape) == (num_pages, nkv, hd, page_size),
-          f"{what}: keys are {tuple(k_pages.shape)}, so values must be {(num_pages, nkv, hd, page_size)}, "
+    _need(page_size % V_GROUP == 0 and tuple(v_pages.shape) == (num_pages, nkv, page_size // V_GROUP, hd, V_GROUP),
+          f"{what}: keys are {tuple(k_pages.shape)}, so values must be "
+          f"{(num_pages, nkv, page_size // V_GROUP, hd, V_GROUP)} with pages a multiple of {V_GROUP}, "
           f"got {tuple(v_pages.shape)}")
     return num_pages, nkv, page_size, hd
 

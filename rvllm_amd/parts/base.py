@@ -88,8 +88,9 @@ CacheNeed = "KVNeed | StateNeed | None"
 class KVCacheView:
     """What an attention-like mixer gets for its layer: the key pages
     ``[num_pages, num_kv_heads, page_size, head_dim]``, the value pages
-    ``[num_pages, num_kv_heads, head_dim, page_size]`` (transposed inside the
-    page) and the name of the group whose block table addresses them.
+    ``[num_pages, num_kv_heads, page_size / 16, head_dim, 16]`` (transposed
+    inside groups of 16 slots: ``csrc/kv_layout.h``) and the name of the group
+    whose block table addresses them.
     ``writes`` is False for a layer that reads another layer's cache."""
 
     k_pages: torch.Tensor

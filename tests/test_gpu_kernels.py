@@ -426,12 +426,15 @@ def paged_setup(T_total, nkv, hd, page_size, dtype, seed, scramble=True):
 def to_cache(k_pages, v_pages):
     """The test keeps pages as [page, slot, kv_head, d]; the cache on the
     device holds keys as [page, kv_head, slot, d] and values transposed inside
-    the page, [page, kv_head, d, slot]."""
-    return dev(k_pages.permute(0, 2, 1, 3)), dev(v_pages.permute(0, 2, 3, 1))
+    groups of 16 slots, [page, kv_head, slot / 16, d, slot % 16]."""
+    n_pages, page_size, nkv, hd = v_pages.shape
+    v = v_pages.view(n_pages, page_size // 16, 16, nkv, hd).permute(0, 3, 1, 4, 2)
+    return dev(k_pages.permute(0, 2, 1, 3)), dev(v)
 
 
 def from_cache(kp, vp):
-    return kp.cpu().permute(0, 2, 1, 3), vp.cpu().permute(0, 3, 1, 2)
+    n_pages, nkv, groups, hd, _ = vp.shape
+    return kp.cpu().permute(0, 2, 1, 3), vp.cpu().permute(0, 2, 4, 1, 3).reshape(n_pages, groups * 16, nkv, hd)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -47,7 +47,8 @@ class LongDecode:
         num_pages = sum(held) + 7
         order = torch.randperm(num_pages, generator=cpu)
         self.k_pages = torch.full((num_pages, nkv, page_size, hd), float("nan"), dtype=torch.bfloat16, device=DEV)
-        self.v_pages = torch.full((num_pages, nkv, hd, page_size), float("nan"), dtype=torch.bfloat16, device=DEV)
+        self.v_pages = torch.full((num_pages, nkv, page_size // 16, hd, 16), float("nan"), dtype=torch.bfloat16,
+                                  device=DEV)  # transposed inside groups of 16 slots
         width = max(-(-L // page_size) for L in self.contexts) + 3
         table = torch.full((B, width), -1, dtype=torch.int32)
         self.keys, self.values, self.first_key = [], [], []
@@ -83,7 +84,7 @@ class LongDecode:
         k = self.keys[b].view(-1, self.page_size, self.nkv, self.hd)
         v = self.values[b].view(-1, self.page_size, self.nkv, self.hd)
         self.k_pages[pages] = k.permute(0, 2, 1, 3)
-        self.v_pages[pages] = v.permute(0, 2, 3, 1)
+        self.v_pages[pages] = v.view(-1, self.page_size // 16, 16, self.nkv, self.hd).permute(0, 3, 1, 4, 2)
 
     def plant(self, b, key, head, dim, value):
         """Key ``key`` of request b becomes ``value`` at one dimension and nothing else."""
