@@ -16,6 +16,7 @@ from typing import Optional
 import torch
 
 from . import build as _build
+from . import signatures as _signatures
 
 _lib = None
 _lock = threading.Lock()
@@ -36,11 +37,11 @@ def library():
             if _lib is None:
                 path = _build.ensure_built()
                 try:
-                    lib = ctypes.CDLL(str(path))
+                    cdll = ctypes.CDLL(str(path))
                 except OSError as e:  # pragma: no cover
                     raise KernelError(f"cannot load the kernel library {path}: {e}") from e
-                lib.rv_last_error.restype = ctypes.c_char_p
-                _lib = lib
+                # every entry point's argument types, from the sources the library was built from
+                _lib = _signatures.Library(cdll, _signatures.read_signatures(_build.CSRC))
     return _lib
 
 
@@ -60,14 +61,17 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _current_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
-def _stream() -> ctypes.c_void_p:
+# The entry points' argument types are declared (``signatures.py``), so a call takes plain numbers: an address as an
+# int or None, a float as a float.  Building a ctypes object for each of the twenty-odd arguments of a launch cost
+# more than the rest of the call.
+def _stream() -> int:
     if _raw_stream is not None and _current_device is not None:
-        return ctypes.c_void_p(_raw_stream(_current_device()))
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        return _raw_stream(_current_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
-def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -94,9 +98,7 @@ def _i32(*tensors: torch.Tensor) -> None:
         _need(t.dtype == torch.int32, f"index tensors must be int32, got {t.dtype}")
 
 
-# A Python int goes to a foreign function as a C int by itself; making a ctypes object for each of the twenty-odd
-# sizes of a launch costs more than the rest of the call.  Floats, 64-bit numbers and addresses keep their types.
-_c_int, _c_float, _c_ll = int, ctypes.c_float, ctypes.c_longlong
+_c_int, _c_float, _c_ll = int, float, int
 
 
 V_GROUP = 16  # slots whose values of one dimension lie side by side (RV_V_GROUP of csrc/kv_layout.h)
@@ -885,7 +887,8 @@ _library_tuning = False
 
 def library_workspace(device) -> torch.Tensor:
     """The device memory that the library's algorithms may use, one allocation a device, made at first use."""
-    index = torch.device(device).index or 0
+    device = torch.device(device)
+    index = torch.cuda.current_device() if device.index is None else device.index
     ws = _library_workspaces.get(index)
     if ws is None:
         ws = _library_workspaces[index] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
@@ -901,17 +904,22 @@ def set_library_tuning(on: bool) -> None:
 
 
 def _library_args(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
-    _need(x.is_cuda and w.is_cuda and out.is_cuda, "library product: arguments must live on the GPU")
-    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
-          "library product: bfloat16 only")
-    _need(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "library product: matrices expected")
     m, k = x.shape
     n = w.shape[0]
-    _need(w.shape[1] == k and out.shape == (m, n), "library product: shapes do not fit")
-    _need(x.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "library product: rows must be contiguous")
-    ws = library_workspace(x.device)
-    return (_ptr(x), _ptr(w), _ptr(out), _c_int(m), _c_int(n), _c_int(k), _c_ll(x.stride(0) if m > 1 else k),
-            _c_ll(w.stride(0) if n > 1 else k), _c_ll(out.stride(0) if m > 1 else n), _ptr(ws), _c_ll(ws.numel()))
+    bf16 = torch.bfloat16
+    if not (x.is_cuda and w.is_cuda and out.is_cuda and x.dtype is bf16 and w.dtype is bf16 and out.dtype is bf16
+            and w.dim() == 2 and w.shape[1] == k and out.dim() == 2 and out.shape[0] == m and out.shape[1] == n
+            and x.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1):
+        _need(x.is_cuda and w.is_cuda and out.is_cuda, "library product: arguments must live on the GPU")
+        _need(x.dtype == bf16 and w.dtype == bf16 and out.dtype == bf16, "library product: bfloat16 only")
+        _need(w.dim() == 2 and out.dim() == 2 and w.shape[1] == k and tuple(out.shape) == (m, n),
+              f"library product: shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+        _need(False, "library product: rows must be contiguous")
+    ws = _library_workspaces.get(x.device.index)
+    if ws is None:
+        ws = library_workspace(x.device)
+    return (x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k, x.stride(0) if m > 1 else k,
+            w.stride(0) if n > 1 else k, out.stride(0) if m > 1 else n, ws.data_ptr(), LIBRARY_WORKSPACE_BYTES)
 
 
 def library_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optional[torch.Tensor]:

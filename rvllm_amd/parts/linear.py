@@ -58,7 +58,16 @@ def linear(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,
     m, k = x.shape
     n = w.shape[0]
     out_dtype = out_dtype or (out.dtype if out is not None else x.dtype)
-    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and m > 0:
+    bf16 = x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16
+    if bf16 and m > ops.SKINNY_MAX_ROWS and out_dtype is torch.bfloat16:
+        # many rows: the library's, on the matrix row by row
+        rows = w.rows if isinstance(w, ops.TiledWeight) else w
+        if rows is not None:
+            if out is None:
+                out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+            if ops.library_gemm(x, rows, out) is not None:
+                return out
+    elif bf16 and m > 0:
         fast = ops.gemm_bf16(x, w, out, out_dtype=out_dtype, sliced_ok=sliced_ok)
         if fast is not None:
             return fast
