@@ -260,7 +260,9 @@ def run_workload(name: str, requests, layers) -> int:
                               max_cache_tokens=sum(lengths) + n_req * (new + 32), use_graphs=True)
     log(f"building the {name}-sized model ({cfg.num_hidden_layers} layers) with random weights")
     engine = LLMEngine.from_random(cfg, 0, engine_cfg)
-    engine.runner.warm_up([portion])
+    t_tune = time.time()
+    ladder = engine.runner.tune_products()  # the library's products tuned at a ladder of row counts up to a step's most
+    log(f"the library's products tuned for {ladder} rows in {time.time() - t_tune:.1f} s")
 
     # What every step of the model must at least do, from the plans the scheduler commits: the bytes it reads
     # (all weights once, the keys and values its tokens may see) and its flops (products, attention, head).

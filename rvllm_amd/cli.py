@@ -14,6 +14,9 @@ ids), ``RVLLM_GEN_PROMPT`` (length of a synthetic prompt), ``RVLLM_GEN_TOKENS``,
 (v3/crates/rvllm-bench/src/main.rs:911-978,1014-1021;
 v3/crates/rvllm-runtime/src/gemma4_bring_up.rs:5594-5611;
 v3/crates/rvllm-serve/src/worker.rs:1171-1181), each also as a flag.
+``--tune-products`` and ``RVLLM_AMD_LIBRARY_PLANS`` (a file of tuned choices, read and written) stand where the
+reference has its autotuned ``RVLLM_POLICY`` file (v3/crates/rvllm-serve/src/main.rs:41): which of the library's
+algorithms a product of a given shape runs on.
 One JSON line per request goes to standard output.
 """
 
@@ -29,7 +32,7 @@ ENV_WHITELIST = {
     "RVLLM_MODEL_DIR", "RVLLM_GEN_PROMPT_FILE", "RVLLM_GEN_PROMPT", "RVLLM_GEN_TOKENS", "RVLLM_GEN_DUMP",
     "RVLLM_SAMPLE_T", "RVLLM_SAMPLE_TOPK", "RVLLM_SAMPLE_TOPP", "RVLLM_SAMPLE_SEED", "RVLLM_EOS",
     "RVLLM_DEFAULT_MAX_TOKENS", "RVLLM_DRY_RUN", "RVLLM_MAX_INFLIGHT_REQUESTS", "RVLLM_DTYPE",
-    "RVLLM_AMD_BUILD_DIR", "RVLLM_GRAPHS",
+    "RVLLM_AMD_BUILD_DIR", "RVLLM_GRAPHS", "RVLLM_AMD_LIBRARY_PLANS", "RVLLM_TUNE_PRODUCTS",
 }
 
 USAGE = """usage: rvllm-amd --model DIR [options]
@@ -53,6 +56,9 @@ USAGE = """usage: rvllm-amd --model DIR [options]
   --random-weights CONFIG.json   no folder: random weights for this configuration (with --weights-seed S)
   --no-graphs                    do not replay decode steps from captured HIP graphs   [$RVLLM_GRAPHS=0]
   --greedy-steps-ahead N         greedy decode steps that may follow one another without the host (default 4, 1 = off)
+  --tune-products                at start-up time the library's algorithms for the products of prompt portions
+                                 and keep the fastest (some seconds)                   [$RVLLM_TUNE_PRODUCTS=1]
+                                 with $RVLLM_AMD_LIBRARY_PLANS=FILE the choices are kept in FILE and read from it
   --dry-run                      check the configuration and the arguments, load nothing
 """
 
@@ -92,6 +98,7 @@ def parse(argv: list[str], env: dict) -> dict:
         "dry_run": env.get("RVLLM_DRY_RUN", "") not in ("", "0", "false"),
         "graphs": env.get("RVLLM_GRAPHS", "1") not in ("0", "false"),
         "greedy_steps_ahead": 4,
+        "tune_products": env.get("RVLLM_TUNE_PRODUCTS", "") not in ("", "0", "false"),
     }
     ints = {"--max-model-len", "--max-num-seqs", "--max-inflight-requests", "--max-num-batched-tokens",
             "--max-prefill-chunk", "--page-size", "--max-cache-tokens", "--prompt-len", "--max-tokens", "--top-k",
@@ -106,7 +113,7 @@ def parse(argv: list[str], env: dict) -> dict:
             raise UsageError(USAGE)
         if key in ("--host", "--port", "--backend", "--served-model-name", "--system-prompt", "--system-prompt-file"):
             raise UsageError(f"{key}: this build has no HTTP server; prompts come from --prompt-file or --prompt-ids")
-        if key in ("--dry-run", "--ignore-eos", "--graphs"):
+        if key in ("--dry-run", "--ignore-eos", "--graphs", "--tune-products"):
             o[key[2:].replace("-", "_")] = True
             continue
         if key == "--no-graphs":
@@ -179,7 +186,8 @@ def main(argv=None, env=None) -> int:
         cfg = EngineConfig(dtype=o["dtype"], page_size=o["page_size"], max_model_len=o["max_model_len"],
                            max_num_seqs=o["max_num_seqs"], max_num_batched_tokens=o["max_num_batched_tokens"],
                            max_prefill_chunk=o["max_prefill_chunk"], max_cache_tokens=o["max_cache_tokens"],
-                           use_graphs=o["graphs"], greedy_steps_ahead=o["greedy_steps_ahead"]).validate()
+                           use_graphs=o["graphs"], greedy_steps_ahead=o["greedy_steps_ahead"],
+                           tune_products=o["tune_products"]).validate()
         if o["random_weights"]:
             doc = json.loads(Path(o["random_weights"]).read_text())
             arch = architecture_of(doc, o["random_weights"])

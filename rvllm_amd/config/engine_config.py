@@ -44,6 +44,11 @@ class EngineConfig:
     # Keep the bf16 matrices a second time, in tiles, for the products of decode steps (up to 64 rows): they then
     # read a matrix as contiguous streams and take a tenth to a quarter less time; the weights take twice the memory.
     tiled_weights: bool = True
+    # At start-up, time the library's algorithms for the products of prompt portions (more than 64 rows) at a ladder
+    # of row counts up to max_num_batched_tokens and keep the fastest (``ModelRunner.tune_products``; some seconds).
+    # Row counts in between run on their tuned neighbour's algorithm.  Off: the library's first suggestion, which
+    # is often a fifth slower.
+    tune_products: bool = False
 
     @property
     def torch_dtype(self) -> torch.dtype:

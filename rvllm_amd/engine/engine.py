@@ -44,6 +44,8 @@ class LLMEngine:
         self.scheduler = Scheduler(runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.max_prefill_chunk,
                                    cfg.max_model_len, on_admit=self._on_admit)
         self.sampler = Sampler(runner.model.spec.vocab_size)
+        if cfg.tune_products and cfg.dtype == "bfloat16":
+            runner.tune_products()
         self._held_back: list[GenerationResult] = []  # results of a step that failed, handed out by the next one
         self.steps = 0
         self.plans = 0  # plans that ran something; fewer than steps when greedy steps followed one another

@@ -249,6 +249,20 @@ class ModelRunner:
         if plans_file:
             ops.library_plans_save(plans_file, self.device)
 
+    def tune_products(self) -> list[int]:
+        """Tunes the library's products (``warm_up``) for a ladder of row counts that the steps of this engine
+        can bring: from just above the few-row kernel's 64 up to ``max_num_batched_tokens``, each one and a half
+        times the one before, and the longest portion of a prompt.  Returns the row counts."""
+        top = min(self.config.max_num_batched_tokens, self.config.max_model_len)
+        rows, n = set(), 96
+        while n < top:
+            rows.add(n)
+            n = n * 3 // 2
+        rows.update(r for r in (top, min(self.config.max_prefill_chunk, top)) if r > ops.SKINNY_MAX_ROWS)
+        ladder = sorted(rows)
+        self.warm_up(ladder)
+        return ladder
+
     # ---- requests ----------------------------------------------------
     def add_request(self, request: Hashable) -> None:
         rc = self.cache.add_request(request)

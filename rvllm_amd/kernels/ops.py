@@ -1008,8 +1008,9 @@ def library_plans_load(path: str, device) -> int:
 
 
 def library_plan_info(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tuple[int, int, float]:
-    """(1 tuned / 0 the library's first suggestion / -1 never seen, the algorithm's index, the time it was tuned
-    to in microseconds) for the shape of this product."""
+    """(1 tuned / 2 a tuned neighbour's algorithm: the nearest row count within one and a half times with the same
+    matrix / 0 the library's first suggestion / -1 never seen, the algorithm's index, the time it was tuned to in
+    microseconds) for the shape of this product."""
     args = _library_args(x, w, out)
     index, us = ctypes.c_int(-1), ctypes.c_float(0.0)
     state = library().rv_lt_plan_info(*args[3:9], ctypes.byref(index), ctypes.byref(us))

@@ -23,6 +23,14 @@ def test_both_spellings_of_a_value_and_the_environment():
     assert cli.parse([], {"RVLLM_MODEL_DIR": "/x"})["model"] == "/x"
 
 
+def test_tuning_of_the_librarys_products_is_asked_for_by_flag_or_environment():
+    assert cli.parse(["--model", "m"], {})["tune_products"] is False
+    assert cli.parse(["--model", "m", "--tune-products"], {})["tune_products"] is True
+    assert cli.parse(["--model", "m"], {"RVLLM_TUNE_PRODUCTS": "1"})["tune_products"] is True
+    assert cli.parse(["--model", "m"], {"RVLLM_TUNE_PRODUCTS": "0"})["tune_products"] is False
+    cli.parse(["--model", "m"], {"RVLLM_AMD_LIBRARY_PLANS": "/tmp/plans.json"})  # a known variable
+
+
 @pytest.mark.parametrize("argv,env,needle", [
     (["--model", "m", "--frobnicate"], {}, "unknown argument: --frobnicate"),
     (["--model", "m"], {"RVLLM_NO_SUCH_THING": "1"}, "unknown environment variable: RVLLM_NO_SUCH_THING"),

@@ -47,6 +47,33 @@ def test_greedy_generation_through_the_python_entry(model_dirs, plain_models, dt
         assert outputs == [plain_gemma.greedy(weights, cfg, p, 12, torch.float64) for p in prompts]
 
 
+def test_generation_with_the_librarys_products_tuned_at_start_up(model_dirs, plain_models, tmp_path, monkeypatch):
+    """``tune_products``: the engine times the library's algorithms for a ladder of row counts before the first
+    request and writes its choices to the file the environment names; a second engine takes them from the file.
+    Prompts of 150 tokens in portions of 100 go through those products; every token is the plain model's."""
+    import json
+
+    from rvllm_amd.kernels import ops
+
+    weights, cfg = plain_models["B"]
+    plans = tmp_path / "plans.json"
+    monkeypatch.setenv(ops.LIBRARY_PLANS_ENV, str(plans))
+    prompts = list(tt.make_sequences(cfg["vocab"], [150, 97], seed=4).values())
+    options = dict(max_tokens=6, dtype="bfloat16", max_model_len=256, max_num_seqs=2, max_num_batched_tokens=160,
+                   max_prefill_chunk=100, tune_products=True)
+    first = rvllm_amd.generate(str(model_dirs["B"]), prompts, **options)
+    for prompt, out in zip(prompts, first):
+        assert_greedy(weights, cfg, prompt, out, "bfloat16")
+    doc = json.loads(plans.read_text())
+    rows = sorted({p[0] for p in doc["plans"]})
+    # the ladder of this engine: 96, 144, the portion, the budget (the file also holds what else this process tuned)
+    assert {96, 100, 144, 160} <= set(rows)
+    again = rvllm_amd.generate(str(model_dirs["B"]), prompts, **options)
+    for prompt, out in zip(prompts, again):
+        assert_greedy(weights, cfg, prompt, out, "bfloat16")
+    assert json.loads(plans.read_text())["plans"] == doc["plans"]  # nothing was tuned again
+
+
 def test_sampled_generation_with_chunked_prompts_is_the_plain_models_stream(model_dirs, plain_models):
     """Workload of the second tiny configuration: six requests with prompts of
     1 to 23 tokens, prompts cut into portions of 7 beside decoding requests,

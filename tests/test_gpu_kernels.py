@@ -359,6 +359,40 @@ def test_the_librarys_product_tuned_gives_the_same_and_keeps_its_plan():
     assert torch.allclose(out.cpu().double(), want, atol=2e-2, rtol=1e-2)
 
 
+def test_a_shape_nobody_tuned_takes_its_tuned_neighbours_algorithm():
+    """A row count that tuning never met runs on the algorithm of the nearest tuned row count with the same matrix
+    (within one and a half times), also when it was first seen before its neighbour was tuned; a row count further
+    off keeps the library's first suggestion.  The results are right whichever algorithm runs."""
+    g = torch.Generator().manual_seed(8)
+    n, k = 448 + 32, 576
+    w = dev((torch.randn(n, k, generator=g) * k ** -0.5).bfloat16())
+
+    def product(m):
+        x = dev(torch.randn(m, k, generator=g).bfloat16())
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+        assert ops.library_gemm(x, w, out) is out
+        assert torch.allclose(out.cpu().double(), x.cpu().double() @ w.cpu().double().T, atol=2e-2, rtol=1e-2), m
+        return ops.library_plan_info(x, w, out)
+
+    early = product(208)  # seen before anything is tuned
+    assert early[0] == 0
+    ops.set_library_tuning(True)
+    try:
+        tuned = product(192)
+    finally:
+        ops.set_library_tuning(False)
+    assert tuned[0] == 1
+    near = product(200)
+    again = product(208)
+    far = product(400)
+    assert far[0] == 0
+    for state, index, _ in (near, again):
+        assert state in (0, 2)  # 0 only if the library says that the algorithm does not take this shape
+        if state == 2:
+            assert index == tuned[1]
+    assert 2 in (near[0], again[0])
+
+
 def test_the_librarys_tuned_plans_go_to_a_file_and_come_back(tmp_path):
     """What tuning found is written as JSON and taken again by index: a plan for a shape this process has not
     seen makes the shape count as tuned (or is refused, if the algorithm does not take the shape) and the product
@@ -405,7 +439,7 @@ def test_the_librarys_tuned_plans_go_to_a_file_and_come_back(tmp_path):
     other.write_text("{ not json")
     assert ops.library_plans_load(str(other), DEV) == 0
     assert ops.library_plans_load(str(tmp_path / "missing.json"), DEV) == 0
-    assert ops.library_plan_info(x3, w, out3)[0] in (-1, 0)
+    assert ops.library_plan_info(x3, w, out3)[0] != 1  # not tuned: unseen, or on its neighbour's algorithm
     assert ops.library_gemm(x3, w, out3) is out3
     assert torch.allclose(out3.cpu().double(), x3.cpu().double() @ w.cpu().double().T, atol=2e-2, rtol=1e-2)
 
