@@ -78,3 +78,52 @@ def test_a_configuration_drawn_at_random_in_every_cutting(tmp_path, seed):
             for rid, logits in got.items():
                 tt.compare(logits, want[rid.split("-", 1)[1]], dtype, f"{what}: {dtype}, {name}, {rid}")
             del runner
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_generation_with_engine_settings_drawn_at_random(tmp_path, seed):
+    """A drawn configuration under drawn engine settings (2 to 6 requests at once, 16 to 200 tokens a step, portions
+    of 7 to 128, pages of 16 to 64, a cache from one request's worth, which sets requests back, to all of them,
+    graphs or none, 1 to 4 greedy steps a plan): 3 to 10 prompts of 1 to 150 tokens, every generated token the plain
+    model's choice, in both dtypes, and no page lost on the way."""
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.engine.engine import LLMEngine
+    from rvllm_amd.models.registry import architecture_of
+    import rvllm_amd.models.gemma3  # noqa: F401
+    from rvllm_amd.sampling.params import SamplingParams
+    from rvllm_amd.weights.random_init import write_random_model
+
+    rng = random.Random(seed)
+    doc = drawn_config(rng)
+    config = architecture_of(doc).read_config(doc, f"drawn configuration {seed}")
+    folder = write_random_model(tmp_path / "model", config, seed, torch.bfloat16)
+    (folder / "config.json").write_text(json.dumps(doc))
+    weights, cfg = plain_gemma.load_weights(folder), plain_gemma.read_config(folder)
+    lengths = [rng.choice([1, 2, 5, 17, 33, 64, 65, 100, 150]) for _ in range(rng.randint(3, 10))]
+    new = rng.choice([4, 9, 20])
+    prompts = list(tt.make_sequences(cfg["vocab"], lengths, seed=seed).values())
+    seqs = rng.randint(2, 6)
+    budget = rng.choice([16, 33, 64, 100, 200])
+    chunk = min(budget, rng.choice([7, 16, 64, 128]))
+    page = rng.choice([16, 32, 64])
+    longest = max(lengths) + new
+    one_request = -(-(longest + 1) // page) * page
+    cache_tokens = rng.choice([one_request + page, 2 * one_request, seqs * one_request])
+    ahead = rng.choice([1, 2, 4])
+    graphs = rng.random() < 0.7
+    what = (f"seed {seed}: {doc}; prompts {lengths} + {new}, {seqs} at once, {budget} tokens a step, portions of "
+            f"{chunk}, pages of {page}, cache {cache_tokens}, {ahead} steps a plan, graphs {graphs}")
+    for dtype in ("float32", "bfloat16"):
+        engine = LLMEngine.from_model_dir(folder, EngineConfig(
+            dtype=dtype, page_size=page, max_model_len=longest + 1, max_num_seqs=seqs, max_num_batched_tokens=budget,
+            max_prefill_chunk=chunk, max_cache_tokens=cache_tokens, use_graphs=graphs, greedy_steps_ahead=ahead))
+        results = engine.generate(prompts, SamplingParams(), new, (), True)
+        for i, (prompt, result) in enumerate(zip(prompts, results)):
+            assert len(result.tokens) == new and result.finish_reason == "length", f"{what}: {dtype}, request {i}"
+            logits = plain_gemma.forward(weights, cfg, (list(prompt) + result.tokens)[:-1], torch.float64)
+            slack = 2 * tt.TOLERANCE[dtype] * logits.abs().max().item()  # a near-tie may fall either way
+            for j, token in enumerate(result.tokens):
+                row = logits[len(prompt) - 1 + j]
+                assert row[token] >= row.max() - slack, f"{what}: {dtype}, request {i}, token {j} is not the arg-max"
+        engine.runner.cache.check()
+        del engine
