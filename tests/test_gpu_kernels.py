@@ -977,6 +977,44 @@ def test_paged_attention_mfma_merges_inside_the_block_only_what_fits():
     assert ops.plan_attention_in_block(1, 8192, 2, None, 256) is None
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_paged_attention_on_batches_drawn_at_random(seed):
+    """Head counts, head sizes, pages, windows and the batch itself drawn at random (decoded tokens only, prompts
+    only, portions deep in a context, or a mix), through ``ops.paged_attention`` left to its own plans: whichever
+    kernels, splits and pieces it takes, the 64-bit reference's output."""
+    import random
+
+    rng = random.Random(seed)
+    nkv, group = rng.choice([1, 2, 3, 4, 8]), rng.choice([1, 2, 3, 4, 5, 8, 16])
+    hd = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 240, 256])
+    page = rng.choice([16, 32, 64])
+    window = rng.choice([None, None, 7, 100, 1024])
+    kind = rng.choice(["decode", "mixed", "prompts", "deep"])
+    portions = []
+    for _ in range(rng.randint(1, 10)):
+        if kind == "decode":
+            portions.append((rng.randint(0, 3000), 1))
+        elif kind == "prompts":
+            portions.append((rng.choice([0, 0, 17, 500]), rng.randint(1, 300)))
+        elif kind == "deep":
+            portions.append((rng.randint(1000, 5000), rng.choice([1, 2, 64, 100, 128])))
+        else:
+            portions.append((rng.randint(0, 2000), rng.choice([1, 1, 1, 2, 3, 40, 64, 65, 130])))
+    if sum(s + n for s, n in portions) * nkv * hd > 6e7:
+        portions = portions[:2]
+    nq = nkv * group
+    case = Case(portions, nq, nkv, hd, page, torch.bfloat16, seed, window)
+    case.step.host_chunk_start = [s for s, _ in portions]
+    case.step.shared = {}
+    T = case.q.shape[0]
+    out = torch.full((T, nq * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    kp, vp = to_cache(case.k_log, case.v_log)
+    ops.paged_attention(dev(case.q.view(T, -1)), kp, vp, dev(case.table), case.step, out, nq, hd ** -0.5, window)
+    got = out.cpu().view(T, nq, hd).float()
+    assert torch.allclose(got, case.reference(hd ** -0.5).float(), **tol(torch.bfloat16)), (
+        f"{nq}:{nkv} heads of {hd}, pages of {page}, window {window}, {kind}: {portions}")
+
+
 def test_paged_attention_mfma_long_decode_batch():
     """Decode shapes: many requests with one token each at long, different contexts."""
     portions = [(4000 + 37 * i, 1) for i in range(9)]
