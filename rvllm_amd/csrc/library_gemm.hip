@@ -12,7 +12,11 @@
 // tensor library's product each call cost 19 us of host time, more than the GPU took for it).  The algorithm is
 // the library's first suggestion unless the shape has been tuned: rv_lt_tune times every algorithm that the
 // library has for the types and that takes the shape (hipblaslt_ext::getAllAlgos, matmulIsAlgoSupported) on the
-// caller's operands and keeps the fastest.  Nothing here allocates device memory: the workspace is the caller's.
+// caller's operands and keeps the fastest; a shape that was never tuned runs on the algorithm of its tuned neighbour
+// in rows (borrow_from_a_neighbour); tuned choices can be listed (rv_lt_tuned_plan) and taken back by their index
+// (rv_lt_take_plan), which is how a file of them survives the process.  Nothing here allocates device memory: the
+// workspace is the caller's.  Calls are serialised by one lock; calls that overlap on a device share the caller's
+// workspace, so they belong on one stream.
 #include <hipblaslt/hipblaslt-ext.hpp>
 #include <hipblaslt/hipblaslt.h>
 
@@ -128,7 +132,19 @@ int plan_for(hipblasLtHandle_t handle, const LtShape& shape, size_t workspace_by
     *out = &it->second;
     return 0;
   }
-  LtPlan plan;
+  // what has been created is given back if the plan is not kept (an error on the way)
+  struct Making {
+    LtPlan plan;
+    bool kept = false;
+    ~Making() {
+      if (kept) return;
+      if (plan.a) hipblasLtMatrixLayoutDestroy(plan.a);
+      if (plan.b) hipblasLtMatrixLayoutDestroy(plan.b);
+      if (plan.d) hipblasLtMatrixLayoutDestroy(plan.d);
+      if (plan.desc) hipblasLtMatmulDescDestroy(plan.desc);
+    }
+  } making;
+  LtPlan& plan = making.plan;
   LT_CHECK(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "hipblasLtMatmulDescCreate");
   const hipblasOperation_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
   LT_CHECK(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_t, sizeof(op_t)), "transpose of w");
@@ -155,6 +171,7 @@ int plan_for(hipblasLtHandle_t handle, const LtShape& shape, size_t workspace_by
   }
   look_for_a_neighbour(handle, shape, workspace_bytes, plan);
   *out = &g_plans.emplace(shape, plan).first->second;
+  making.kept = true;
   return 0;
 }
 
@@ -218,9 +235,18 @@ extern "C" int rv_lt_tune(hipStream_t stream, const void* x, const void* w, void
                                       HIP_R_16BF, HIP_R_16BF, HIP_R_16BF, HIP_R_16BF, HIPBLAS_COMPUTE_32F, all),
            "getAllAlgos");
   const float one = 1.f, zero = 0.f;
-  hipEvent_t t0, t1, begin;
-  RV_CHECK(hipEventCreate(&t0) == hipSuccess && hipEventCreate(&t1) == hipSuccess && hipEventCreate(&begin) == hipSuccess,
+  struct Events {
+    hipEvent_t t0 = nullptr, t1 = nullptr, begin = nullptr;
+    ~Events() {
+      if (t0) hipEventDestroy(t0);
+      if (t1) hipEventDestroy(t1);
+      if (begin) hipEventDestroy(begin);
+    }
+  } events;
+  RV_CHECK(hipEventCreate(&events.t0) == hipSuccess && hipEventCreate(&events.t1) == hipSuccess &&
+               hipEventCreate(&events.begin) == hipSuccess,
            "library product: hipEventCreate failed");
+  const hipEvent_t t0 = events.t0, t1 = events.t1, begin = events.begin;
   auto run = [&](hipblasLtMatmulAlgo_t& algo, size_t ws) {
     return hipblasLtMatmul(handle, plan->desc, &one, w, plan->a, x, plan->b, &zero, out, plan->d, out, plan->d, &algo,
                            workspace, ws, stream);
@@ -279,9 +305,6 @@ extern "C" int rv_lt_tune(hipStream_t stream, const void* x, const void* w, void
       plan->algo_index = hipblaslt_ext::getIndexFromAlgo(all[i].algo);
     }
   }
-  hipEventDestroy(t0);
-  hipEventDestroy(t1);
-  hipEventDestroy(begin);
   RV_CHECK(best_us > 0.f, "library product: no algorithm ran for M=%d N=%d K=%d", M, N, K);
   plan->tuned = true;
   plan->tuned_us = best_us;
