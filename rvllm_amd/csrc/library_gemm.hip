@@ -218,9 +218,13 @@ extern "C" int rv_lt_gemm(hipStream_t stream, const void* x, const void* w, void
 // Times every algorithm the library has for this shape on the given operands (their contents do not matter; `out`
 // is overwritten) and keeps the fastest for rv_lt_gemm.  Waits for the device.  Returns the number of algorithms
 // timed, or -1; a shape that was tuned before returns 0 at once.  `budget_ms` bounds the time spent.
+// `w_others` (num_others of them, may be none): other matrices of the same shape and stride, a model's other layers'.
+// The timed calls then take them in turn, so that a call reads its matrix from memory as a step's calls do, layer
+// after layer, and not from the cache that the same matrix called over and over would stay in: the algorithm that
+// is fastest on a matrix in the cache is not always the one that streams it fastest.
 extern "C" int rv_lt_tune(hipStream_t stream, const void* x, const void* w, void* out, int M, int N, int K,
                           long long ldx, long long ldw, long long ldc, void* workspace, long long workspace_bytes,
-                          int budget_ms) {
+                          int budget_ms, const void* const* w_others, int num_others) {
   if (check_operands(x, w, out, M, N, K, ldx, ldw, ldc)) return -1;
   int dev = 0;
   RV_CHECK(hipGetDevice(&dev) == hipSuccess, "library product: no current device");
@@ -247,9 +251,12 @@ extern "C" int rv_lt_tune(hipStream_t stream, const void* x, const void* w, void
                hipEventCreate(&events.begin) == hipSuccess,
            "library product: hipEventCreate failed");
   const hipEvent_t t0 = events.t0, t1 = events.t1, begin = events.begin;
+  RV_CHECK(num_others >= 0 && (num_others == 0 || w_others), "library product: bad list of other matrices");
+  long long turn = 0;
   auto run = [&](hipblasLtMatmulAlgo_t& algo, size_t ws) {
-    return hipblasLtMatmul(handle, plan->desc, &one, w, plan->a, x, plan->b, &zero, out, plan->d, out, plan->d, &algo,
-                           workspace, ws, stream);
+    const void* w_now = num_others > 0 ? w_others[turn++ % num_others] : w;
+    return hipblasLtMatmul(handle, plan->desc, &one, w_now, plan->a, x, plan->b, &zero, out, plan->d, out, plan->d,
+                           &algo, workspace, ws, stream);
   };
   // the time of `runs` calls in a row, per call (microseconds); negative if a call failed
   auto time_of = [&](hipblasLtMatmulAlgo_t& algo, size_t ws, int runs) -> float {

@@ -922,6 +922,33 @@ def _library_args(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
             w.stride(0) if n > 1 else k, out.stride(0) if m > 1 else n, ws.data_ptr(), LIBRARY_WORKSPACE_BYTES)
 
 
+# The matrices that products of many rows may meet, by shape: tuning a shape takes them in turn (``rv_lt_tune``), so
+# that its timed calls read from memory as a step's calls do.  Weak references: a model that goes takes its own along.
+_library_matrices: dict = {}
+
+
+def library_matrix_register(w: torch.Tensor) -> None:
+    """Tells the tuning of the library's products that ``w`` ([N, K], bf16, on the GPU) is one of the matrices of
+    its shape: a part calls it for every matrix it keeps row by row."""
+    import weakref
+
+    if w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.stride(1) == 1:
+        key = (w.device.index, w.shape[0], w.shape[1], w.stride(0))
+        _library_matrices.setdefault(key, []).append(weakref.ref(w))
+
+
+def _library_matrices_like(w: torch.Tensor):
+    """(a C array of the addresses of the registered matrices of ``w``'s shape that are still there, their number);
+    (None, 0) if there is none but ``w`` itself."""
+    key = (w.device.index, w.shape[0], w.shape[1], w.stride(0))
+    alive = [t for t in (ref() for ref in _library_matrices.get(key, ())) if t is not None]
+    _library_matrices[key] = [ref for ref in _library_matrices.get(key, ()) if ref() is not None]
+    addresses = sorted({t.data_ptr() for t in alive} | {w.data_ptr()})
+    if len(addresses) < 2:
+        return None, 0
+    return (ctypes.c_void_p * len(addresses))(*addresses), len(addresses)
+
+
 def library_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optional[torch.Tensor]:
     """out[M, N] = x[M, K] @ w[N, K]^T in bf16 with 32-bit sums, by hipBLASLt (``csrc/library_gemm.hip``): the
     product of more rows than the few-row kernel takes.  A shape keeps its plan; see ``set_library_tuning``.
@@ -929,7 +956,8 @@ def library_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optiona
     args = _library_args(x, w, out)
     lib = library()
     if _library_tuning:
-        _check(min(0, lib.rv_lt_tune(_stream(), *args, _c_int(LIBRARY_TUNE_BUDGET_MS))))
+        others, count = _library_matrices_like(w)
+        _check(min(0, lib.rv_lt_tune(_stream(), *args, _c_int(LIBRARY_TUNE_BUDGET_MS), others, _c_int(count))))
     status = lib.rv_lt_gemm(_stream(), *args)
     if status == 2:  # the library has no algorithm for this shape: nothing ran
         return None

@@ -23,8 +23,11 @@ def decode_weight(w: torch.Tensor, tiled: bool = True):
     is the engine's setting) a bf16 matrix on the GPU goes into tiles for the few-row product
     (``ops.TiledWeight``; the matrix row by row is kept beside the tiles for the products that go to the
     library), anything else stays as it is."""
-    if tiled and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2:
-        return ops.TiledWeight(w.contiguous())
+    if w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2:
+        w = w.contiguous()
+        ops.library_matrix_register(w)  # the tuning of the products of many rows takes a shape's matrices in turn
+        if tiled:
+            return ops.TiledWeight(w)
     return w
 
 
