@@ -934,7 +934,10 @@ def library_matrix_register(w: torch.Tensor) -> None:
 
     if w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.stride(1) == 1:
         key = (w.device.index, w.shape[0], w.shape[1], w.stride(0))
-        _library_matrices.setdefault(key, []).append(weakref.ref(w))
+        known = _library_matrices.setdefault(key, [])
+        if len(known) >= 1024:  # models come and go: forget the ones that went
+            known[:] = [ref for ref in known if ref() is not None]
+        known.append(weakref.ref(w))
 
 
 def _library_matrices_like(w: torch.Tensor):
