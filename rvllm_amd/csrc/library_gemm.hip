@@ -2,7 +2,8 @@
 // hipBLASLt, as the reference hands its products to cuBLASLt (v3/crates/rvllm-cutlass/src/cublaslt.rs:184-277:
 // one descriptor set and one chosen algorithm per shape, a workspace the caller owns).
 //
-//   out[M, N] (bf16, row stride ldc) = x[M, K] (row stride ldx) * w[N, K]^T (row stride ldw), sums in 32 bits.
+//   out[M, N] (bf16, or 32-bit with out_f32: logits; row stride ldc) = x[M, K] (row stride ldx) * w[N, K]^T (row
+//   stride ldw), x and w in bf16, sums in 32 bits.
 //
 // The library counts in columns: the row-major out[M, N] is its column-major [N, M], so the call is
 // D(N x M) = op_T(A = w as K x N) * (B = x as K x M).
@@ -34,8 +35,9 @@ namespace {
 struct LtShape {
   int dev, M, N, K;
   long long ldx, ldw, ldc;
+  int out_f32;  // the result is stored in 32 bits (logits) instead of bf16
   bool operator<(const LtShape& o) const {
-    return std::tie(dev, M, N, K, ldx, ldw, ldc) < std::tie(o.dev, o.M, o.N, o.K, o.ldx, o.ldw, o.ldc);
+    return std::tie(dev, M, N, K, ldx, ldw, ldc, out_f32) < std::tie(o.dev, o.M, o.N, o.K, o.ldx, o.ldw, o.ldc, o.out_f32);
   }
 };
 
@@ -98,7 +100,7 @@ void borrow_from_a_neighbour(hipblasLtHandle_t handle, const LtShape& shape, siz
   double nearest_ratio = RV_LT_NEIGHBOUR;
   for (const auto& kv : g_plans) {
     const LtShape& o = kv.first;
-    if (o.dev != shape.dev || o.N != shape.N || o.K != shape.K || o.ldw != shape.ldw) continue;
+    if (o.dev != shape.dev || o.N != shape.N || o.K != shape.K || o.ldw != shape.ldw || o.out_f32 != shape.out_f32) continue;
     if (!kv.second.tuned || kv.second.none) continue;
     const double ratio = o.M > shape.M ? (double)o.M / shape.M : (double)shape.M / o.M;
     if (ratio <= nearest_ratio) nearest = &kv.second, nearest_rows = o.M, nearest_ratio = ratio;
@@ -152,7 +154,8 @@ int plan_for(hipblasLtHandle_t handle, const LtShape& shape, size_t workspace_by
   // as stored (before the transposition): w is K x N in columns, x is K x M, out is N x M
   LT_CHECK(hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, shape.K, shape.N, shape.ldw), "layout of w");
   LT_CHECK(hipblasLtMatrixLayoutCreate(&plan.b, HIP_R_16BF, shape.K, shape.M, shape.ldx), "layout of x");
-  LT_CHECK(hipblasLtMatrixLayoutCreate(&plan.d, HIP_R_16BF, shape.N, shape.M, shape.ldc), "layout of out");
+  LT_CHECK(hipblasLtMatrixLayoutCreate(&plan.d, shape.out_f32 ? HIP_R_32F : HIP_R_16BF, shape.N, shape.M, shape.ldc),
+           "layout of out");
   hipblasLtMatmulPreference_t pref = nullptr;
   LT_CHECK(hipblasLtMatmulPreferenceCreate(&pref), "hipblasLtMatmulPreferenceCreate");
   const uint64_t room = workspace_bytes;
@@ -192,7 +195,8 @@ int check_operands(const void* x, const void* w, void* out, int M, int N, int K,
 
 // out = x w^T on `stream`; 0, RV_LT_NO_ALGORITHM or -1 (an error); `workspace` (workspace_bytes of device memory, the caller's) is what the algorithm may use.
 extern "C" int rv_lt_gemm(hipStream_t stream, const void* x, const void* w, void* out, int M, int N, int K,
-                          long long ldx, long long ldw, long long ldc, void* workspace, long long workspace_bytes) {
+                          long long ldx, long long ldw, long long ldc, void* workspace, long long workspace_bytes,
+                          int out_f32) {
   if (check_operands(x, w, out, M, N, K, ldx, ldw, ldc)) return -1;
   int dev = 0;
   RV_CHECK(hipGetDevice(&dev) == hipSuccess, "library product: no current device");
@@ -200,7 +204,7 @@ extern "C" int rv_lt_gemm(hipStream_t stream, const void* x, const void* w, void
   hipblasLtHandle_t handle;
   if (handle_for(dev, &handle)) return -1;
   LtPlan* plan;
-  if (plan_for(handle, LtShape{dev, M, N, K, ldx, ldw, ldc}, (size_t)workspace_bytes, &plan)) return -1;
+  if (plan_for(handle, LtShape{dev, M, N, K, ldx, ldw, ldc, out_f32 != 0}, (size_t)workspace_bytes, &plan)) return -1;
   if (plan->none) {
     rv_fail("library product: the library has no algorithm for M=%d N=%d K=%d (strides %lld %lld %lld)", M, N, K, ldx,
             ldw, ldc);
@@ -224,7 +228,7 @@ extern "C" int rv_lt_gemm(hipStream_t stream, const void* x, const void* w, void
 // is fastest on a matrix in the cache is not always the one that streams it fastest.
 extern "C" int rv_lt_tune(hipStream_t stream, const void* x, const void* w, void* out, int M, int N, int K,
                           long long ldx, long long ldw, long long ldc, void* workspace, long long workspace_bytes,
-                          int budget_ms, const void* const* w_others, int num_others) {
+                          int budget_ms, const void* const* w_others, int num_others, int out_f32) {
   if (check_operands(x, w, out, M, N, K, ldx, ldw, ldc)) return -1;
   int dev = 0;
   RV_CHECK(hipGetDevice(&dev) == hipSuccess, "library product: no current device");
@@ -232,11 +236,12 @@ extern "C" int rv_lt_tune(hipStream_t stream, const void* x, const void* w, void
   hipblasLtHandle_t handle;
   if (handle_for(dev, &handle)) return -1;
   LtPlan* plan;
-  if (plan_for(handle, LtShape{dev, M, N, K, ldx, ldw, ldc}, (size_t)workspace_bytes, &plan)) return -1;
+  if (plan_for(handle, LtShape{dev, M, N, K, ldx, ldw, ldc, out_f32 != 0}, (size_t)workspace_bytes, &plan)) return -1;
   if (plan->tuned || plan->none) return 0;
   std::vector<hipblasLtMatmulHeuristicResult_t> all;
   LT_CHECK(hipblaslt_ext::getAllAlgos(handle, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, HIPBLAS_OP_T, HIPBLAS_OP_N,
-                                      HIP_R_16BF, HIP_R_16BF, HIP_R_16BF, HIP_R_16BF, HIPBLAS_COMPUTE_32F, all),
+                                      HIP_R_16BF, HIP_R_16BF, out_f32 ? HIP_R_32F : HIP_R_16BF,
+                                      out_f32 ? HIP_R_32F : HIP_R_16BF, HIPBLAS_COMPUTE_32F, all),
            "getAllAlgos");
   const float one = 1.f, zero = 0.f;
   struct Events {
@@ -322,11 +327,11 @@ extern "C" int rv_lt_tune(hipStream_t stream, const void* x, const void* w, void
 // What is kept for a shape: 1 if it has been tuned, 2 if it runs on a tuned neighbour's algorithm, 0 if it runs on the
 // library's first suggestion, -1 if it has not been seen; the algorithm's index in the library and the time it was tuned to (microseconds) if asked for.
 extern "C" int rv_lt_plan_info(int M, int N, int K, long long ldx, long long ldw, long long ldc, int* algo_index,
-                               float* tuned_us) {
+                               float* tuned_us, int out_f32) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return -1;
   std::lock_guard<std::mutex> guard(g_lock);
-  auto it = g_plans.find(LtShape{dev, M, N, K, ldx, ldw, ldc});
+  auto it = g_plans.find(LtShape{dev, M, N, K, ldx, ldw, ldc, out_f32 != 0});
   if (it == g_plans.end()) return -1;
   if (algo_index) *algo_index = it->second.algo_index;
   if (tuned_us) *tuned_us = it->second.tuned_us;
@@ -362,7 +367,7 @@ extern "C" int rv_lt_device_kind(char* out, int room) {
 // The `i`-th tuned shape of the current device, in no particular order: 1 and the shape, its algorithm's index and
 // its time; 0 when there are fewer.
 extern "C" int rv_lt_tuned_plan(int i, int* M, int* N, int* K, long long* ldx, long long* ldw, long long* ldc,
-                                int* algo_index, float* tuned_us) {
+                                int* algo_index, float* tuned_us, int* out_f32) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   std::lock_guard<std::mutex> guard(g_lock);
@@ -373,6 +378,7 @@ extern "C" int rv_lt_tuned_plan(int i, int* M, int* N, int* K, long long* ldx, l
     *ldx = kv.first.ldx, *ldw = kv.first.ldw, *ldc = kv.first.ldc;
     *algo_index = kv.second.algo_index;
     *tuned_us = kv.second.tuned_us;
+    *out_f32 = kv.first.out_f32;
     return 1;
   }
   return 0;
@@ -383,7 +389,7 @@ extern "C" int rv_lt_tuned_plan(int i, int* M, int* N, int* K, long long* ldx, l
 // or the algorithm does not take the shape (nothing changes: the shape runs on the first suggestion and can be
 // tuned), -1 on an error.
 extern "C" int rv_lt_take_plan(int M, int N, int K, long long ldx, long long ldw, long long ldc, int algo_index,
-                               float tuned_us, long long workspace_bytes) {
+                               float tuned_us, long long workspace_bytes, int out_f32) {
   RV_CHECK(M > 0 && N > 0 && K > 0 && ldx >= K && ldw >= K && ldc >= N && algo_index >= 0,
            "library product: bad plan M=%d N=%d K=%d index=%d", M, N, K, algo_index);
   int dev = 0;
@@ -392,7 +398,7 @@ extern "C" int rv_lt_take_plan(int M, int N, int K, long long ldx, long long ldw
   hipblasLtHandle_t handle;
   if (handle_for(dev, &handle)) return -1;
   LtPlan* plan;
-  if (plan_for(handle, LtShape{dev, M, N, K, ldx, ldw, ldc}, (size_t)workspace_bytes, &plan)) return -1;
+  if (plan_for(handle, LtShape{dev, M, N, K, ldx, ldw, ldc, out_f32 != 0}, (size_t)workspace_bytes, &plan)) return -1;
   if (plan->tuned) return 0;
   if (plan->none) return RV_LT_NO_ALGORITHM;
   std::vector<int> wanted{algo_index};

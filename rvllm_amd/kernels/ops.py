@@ -907,11 +907,14 @@ def _library_args(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
     m, k = x.shape
     n = w.shape[0]
     bf16 = torch.bfloat16
-    if not (x.is_cuda and w.is_cuda and out.is_cuda and x.dtype is bf16 and w.dtype is bf16 and out.dtype is bf16
+    out_f32 = out.dtype is torch.float32
+    if not (x.is_cuda and w.is_cuda and out.is_cuda and x.dtype is bf16 and w.dtype is bf16
+            and (out.dtype is bf16 or out_f32)
             and w.dim() == 2 and w.shape[1] == k and out.dim() == 2 and out.shape[0] == m and out.shape[1] == n
             and x.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1):
         _need(x.is_cuda and w.is_cuda and out.is_cuda, "library product: arguments must live on the GPU")
-        _need(x.dtype == bf16 and w.dtype == bf16 and out.dtype == bf16, "library product: bfloat16 only")
+        _need(x.dtype == bf16 and w.dtype == bf16 and out.dtype in (bf16, torch.float32),
+              "library product: bfloat16 operands, a bfloat16 or float32 result")
         _need(w.dim() == 2 and out.dim() == 2 and w.shape[1] == k and tuple(out.shape) == (m, n),
               f"library product: shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
         _need(False, "library product: rows must be contiguous")
@@ -919,7 +922,7 @@ def _library_args(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
     if ws is None:
         ws = library_workspace(x.device)
     return (x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k, x.stride(0) if m > 1 else k,
-            w.stride(0) if n > 1 else k, out.stride(0) if m > 1 else n, ws.data_ptr(), LIBRARY_WORKSPACE_BYTES)
+            w.stride(0) if n > 1 else k, out.stride(0) if m > 1 else n, ws.data_ptr(), LIBRARY_WORKSPACE_BYTES), int(out_f32)
 
 
 # The matrices that products of many rows may meet, by shape: tuning a shape takes them in turn (``rv_lt_tune``), so
@@ -953,15 +956,15 @@ def _library_matrices_like(w: torch.Tensor):
 
 
 def library_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Optional[torch.Tensor]:
-    """out[M, N] = x[M, K] @ w[N, K]^T in bf16 with 32-bit sums, by hipBLASLt (``csrc/library_gemm.hip``): the
-    product of more rows than the few-row kernel takes.  A shape keeps its plan; see ``set_library_tuning``.
+    """out[M, N] = x[M, K] @ w[N, K]^T, x and w in bf16, out in bf16 or (logits) float32, with 32-bit sums, by
+    hipBLASLt (``csrc/library_gemm.hip``): the product of more rows than the few-row kernel takes.  A shape keeps its plan; see ``set_library_tuning``.
     None, with nothing done, for a shape that the library has no algorithm for."""
-    args = _library_args(x, w, out)
+    args, out_f32 = _library_args(x, w, out)
     lib = library()
     if _library_tuning:
         others, count = _library_matrices_like(w)
-        _check(min(0, lib.rv_lt_tune(_stream(), *args, _c_int(LIBRARY_TUNE_BUDGET_MS), others, _c_int(count))))
-    status = lib.rv_lt_gemm(_stream(), *args)
+        _check(min(0, lib.rv_lt_tune(_stream(), *args, _c_int(LIBRARY_TUNE_BUDGET_MS), others, _c_int(count), out_f32)))
+    status = lib.rv_lt_gemm(_stream(), *args, out_f32)
     if status == 2:  # the library has no algorithm for this shape: nothing ran
         return None
     _check(status)
@@ -984,7 +987,7 @@ def _library_plans_key(device) -> dict:
 
 
 def library_plans_save(path: str, device) -> int:
-    """Writes the tuned shapes of ``device`` (shape, strides, the algorithm's index, its time) to ``path`` as JSON,
+    """Writes the tuned shapes of ``device`` (shape, strides, the algorithm's index, its time, 1 for a 32-bit result) to ``path`` as JSON,
     over what the file held; the number of shapes written."""
     import json
     import os
@@ -993,14 +996,15 @@ def library_plans_save(path: str, device) -> int:
     plans = []
     with torch.cuda.device(device):
         while True:
-            m, n, k, index = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+            m, n, k, index, f32 = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
             ldx, ldw, ldc = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_longlong()
             us = ctypes.c_float()
             if not lib.rv_lt_tuned_plan(_c_int(len(plans)), ctypes.byref(m), ctypes.byref(n), ctypes.byref(k),
                                         ctypes.byref(ldx), ctypes.byref(ldw), ctypes.byref(ldc), ctypes.byref(index),
-                                        ctypes.byref(us)):
+                                        ctypes.byref(us), ctypes.byref(f32)):
                 break
-            plans.append([m.value, n.value, k.value, ldx.value, ldw.value, ldc.value, index.value, round(us.value, 2)])
+            plans.append([m.value, n.value, k.value, ldx.value, ldw.value, ldc.value, index.value, round(us.value, 2),
+                          f32.value])
         doc = dict(_library_plans_key(device), plans=sorted(plans))
     tmp = f"{path}.{os.getpid()}.tmp"
     with open(tmp, "w") as f:
@@ -1018,8 +1022,8 @@ def library_plans_load(path: str, device) -> int:
     try:
         with open(path) as f:
             doc = json.load(f)
-        plans = [(int(m), int(n), int(k), int(ldx), int(ldw), int(ldc), int(index), float(us))
-                 for m, n, k, ldx, ldw, ldc, index, us in doc["plans"]]
+        plans = [(int(m), int(n), int(k), int(ldx), int(ldw), int(ldc), int(index), float(us), int(f32))
+                 for m, n, k, ldx, ldw, ldc, index, us, f32 in doc["plans"]]
     except (OSError, ValueError, KeyError, TypeError):
         return 0
     lib = library()
@@ -1028,9 +1032,9 @@ def library_plans_load(path: str, device) -> int:
         if {key: doc.get(key) for key in ("device", "hipblaslt")} != _library_plans_key(device):
             return 0
         room = library_workspace(torch.device(device)).numel()
-        for m, n, k, ldx, ldw, ldc, index, us in plans:
+        for m, n, k, ldx, ldw, ldc, index, us, f32 in plans:
             status = lib.rv_lt_take_plan(_c_int(m), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(ldc),
-                                         _c_int(index), _c_float(us), _c_ll(room))
+                                         _c_int(index), _c_float(us), _c_ll(room), _c_int(f32))
             if status == 0:
                 taken += 1
             elif status != 2:
@@ -1042,9 +1046,9 @@ def library_plan_info(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> tu
     """(1 tuned / 2 a tuned neighbour's algorithm: the nearest row count within one and a half times with the same
     matrix / 0 the library's first suggestion / -1 never seen, the algorithm's index, the time it was tuned to in
     microseconds) for the shape of this product."""
-    args = _library_args(x, w, out)
+    args, out_f32 = _library_args(x, w, out)
     index, us = ctypes.c_int(-1), ctypes.c_float(0.0)
-    state = library().rv_lt_plan_info(*args[3:9], ctypes.byref(index), ctypes.byref(us))
+    state = library().rv_lt_plan_info(*args[3:9], ctypes.byref(index), ctypes.byref(us), out_f32)
     return state, index.value, us.value
 
 

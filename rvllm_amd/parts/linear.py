@@ -62,7 +62,7 @@ def linear(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,
     n = w.shape[0]
     out_dtype = out_dtype or (out.dtype if out is not None else x.dtype)
     bf16 = x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16
-    if bf16 and m > ops.SKINNY_MAX_ROWS and out_dtype is torch.bfloat16:
+    if bf16 and m > ops.SKINNY_MAX_ROWS and out_dtype in (torch.bfloat16, torch.float32):
         # many rows: the library's, on the matrix row by row
         rows = w.rows if isinstance(w, ops.TiledWeight) else w
         if rows is not None:
@@ -70,6 +70,10 @@ def linear(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,
                 out = torch.empty((m, n), dtype=out_dtype, device=x.device)
             if ops.library_gemm(x, rows, out) is not None:
                 return out
+        if out_dtype is torch.float32:  # no algorithm: the few-row kernel, 64 rows at a time
+            fast = ops.gemm_bf16(x, w, out, out_dtype=out_dtype, sliced_ok=sliced_ok)
+            if fast is not None:
+                return fast
     elif bf16 and m > 0:
         fast = ops.gemm_bf16(x, w, out, out_dtype=out_dtype, sliced_ok=sliced_ok)
         if fast is not None:

@@ -334,6 +334,29 @@ def test_the_librarys_product_against_64_bit(m, n, k):
     assert bool((wide_out[:, :16] == 7.0).all()) and bool((wide_out[:, 16 + n:] == 7.0).all())
 
 
+@pytest.mark.parametrize("m,n,k", [(65, 1000, 128), (200, 4096 + 64, 2560), (130, 333, 72)])
+def test_the_librarys_product_with_a_32_bit_result(m, n, k):
+    """Logits at many positions: bf16 operands, the sums stored in 32 bits, unrounded; through ``linear`` whichever
+    kernel takes the shape."""
+    from rvllm_amd.parts.linear import linear
+
+    g = torch.Generator().manual_seed(m * n + k)
+    x = dev(torch.randn(m, k, generator=g).bfloat16())
+    w = dev((torch.randn(n, k, generator=g) * k ** -0.5).bfloat16())
+    want = x.cpu().double() @ w.cpu().double().T
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+    got = ops.library_gemm(x, w, out)
+    if got is None:
+        assert bool(torch.isnan(out).all())
+    else:
+        assert torch.allclose(out.cpu().double(), want, atol=1e-4, rtol=1e-4)  # no rounding to bf16 at the end
+        assert ops.library_plan_info(x, w, out)[0] in (0, 2)
+        assert ops.library_plan_info(x, w, torch.empty((m, n), dtype=torch.bfloat16, device=DEV))[0] in (-1, 0, 2)
+    logits = linear(x, ops.TiledWeight(w), out_dtype=torch.float32)
+    assert logits.dtype == torch.float32
+    assert torch.allclose(logits.cpu().double(), want, atol=1e-4, rtol=1e-4)
+
+
 def test_the_librarys_product_tuned_gives_the_same_and_keeps_its_plan():
     g = torch.Generator().manual_seed(5)
     m, n, k = 160, 512 + 32, 640
@@ -414,7 +437,7 @@ def test_the_librarys_tuned_plans_go_to_a_file_and_come_back(tmp_path):
     path = tmp_path / "plans.json"
     assert ops.library_plans_save(str(path), DEV) >= 1
     doc = json.loads(path.read_text())
-    assert [m, n, k, k, k, n, index] in [p[:7] for p in doc["plans"]]
+    assert [m, n, k, k, k, n, index, 0] in [p[:7] + p[8:] for p in doc["plans"]]  # the last field: a bf16 result
     assert ops.library_plans_load(str(path), DEV) == len(doc["plans"])  # all known already: they stay as they are
 
     m2 = m + 16  # a shape nobody has tuned here, under the first one's algorithm
@@ -422,7 +445,7 @@ def test_the_librarys_tuned_plans_go_to_a_file_and_come_back(tmp_path):
     out2 = torch.empty((m2, n), dtype=torch.bfloat16, device=DEV)
     assert ops.library_plan_info(x2, w, out2)[0] == -1
     other = tmp_path / "other.json"
-    other.write_text(json.dumps(dict(doc, plans=[[m2, n, k, k, k, n, index, 12.5]])))
+    other.write_text(json.dumps(dict(doc, plans=[[m2, n, k, k, k, n, index, 12.5, 0]])))
     taken = ops.library_plans_load(str(other), DEV)
     assert taken in (0, 1)
     assert ops.library_plan_info(x2, w, out2)[:2] == ((1, index) if taken else (0, ops.library_plan_info(x2, w, out2)[1]))
@@ -432,9 +455,9 @@ def test_the_librarys_tuned_plans_go_to_a_file_and_come_back(tmp_path):
     m3 = m + 32
     x3 = dev(torch.randn(m3, k, generator=g).bfloat16())
     out3 = torch.empty((m3, n), dtype=torch.bfloat16, device=DEV)
-    other.write_text(json.dumps(dict(doc, hipblaslt=doc["hipblaslt"] + 1, plans=[[m3, n, k, k, k, n, index, 12.5]])))
+    other.write_text(json.dumps(dict(doc, hipblaslt=doc["hipblaslt"] + 1, plans=[[m3, n, k, k, k, n, index, 12.5, 0]])))
     assert ops.library_plans_load(str(other), DEV) == 0
-    other.write_text(json.dumps(dict(doc, plans=[[m3, n, k, k, k, n, 1 << 30, 12.5]])))  # no such algorithm
+    other.write_text(json.dumps(dict(doc, plans=[[m3, n, k, k, k, n, 1 << 30, 12.5, 0]])))  # no such algorithm
     assert ops.library_plans_load(str(other), DEV) == 0
     other.write_text("{ not json")
     assert ops.library_plans_load(str(other), DEV) == 0
