@@ -240,7 +240,10 @@ class ModelRunner:
                     continue
                 self.add_request("__warm_up__")
                 try:
-                    self.step([("__warm_up__", [0] * n, [n - 1])])
+                    # as many rows as requests may decode together want their logits, as such a decode step does:
+                    # the head's product of that many rows is then met (and tuned) too
+                    wanted = list(range(n)) if n <= self.config.max_num_seqs else [n - 1]
+                    self.step([("__warm_up__", [0] * n, wanted)])
                 finally:
                     self.release("__warm_up__")
             torch.cuda.synchronize(self.device)
