@@ -250,7 +250,10 @@ class ModelRunner:
         finally:
             ops.set_library_tuning(False)
         if plans_file:
-            ops.library_plans_save(plans_file, self.device)
+            try:
+                ops.library_plans_save(plans_file, self.device)
+            except OSError as e:  # a place that cannot be written costs the next start its tuning, not this one its work
+                warnings.warn(f"the tuned plans were not written to {plans_file}: {e}")
 
     def tune_products(self) -> list[int]:
         """Tunes the library's products (``warm_up``) for a ladder of row counts that the steps of this engine

@@ -72,6 +72,10 @@ def test_generation_with_the_librarys_products_tuned_at_start_up(model_dirs, pla
     for prompt, out in zip(prompts, again):
         assert_greedy(weights, cfg, prompt, out, "bfloat16")
     assert json.loads(plans.read_text())["plans"] == doc["plans"]  # nothing was tuned again
+    # a file that cannot be written is a warning, not an error
+    monkeypatch.setenv(ops.LIBRARY_PLANS_ENV, str(tmp_path / "no" / "such" / "folder" / "plans.json"))
+    with pytest.warns(UserWarning, match="were not written"):
+        rvllm_amd.generate(str(model_dirs["B"]), prompts[:1], **options)
 
 
 def test_sampled_generation_with_chunked_prompts_is_the_plain_models_stream(model_dirs, plain_models):
