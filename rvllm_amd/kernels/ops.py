@@ -1036,9 +1036,7 @@ def library_plans_load(path: str, device) -> int:
             status = lib.rv_lt_take_plan(_c_int(m), _c_int(n), _c_int(k), _c_ll(ldx), _c_ll(ldw), _c_ll(ldc),
                                          _c_int(index), _c_float(us), _c_ll(room), _c_int(f32))
             if status == 0:
-                taken += 1
-            elif status != 2:
-                _check(status)
+                taken += 1  # anything else: the library does not know the algorithm, or refuses the shape; not taken
     return taken
 
 

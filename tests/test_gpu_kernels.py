@@ -459,6 +459,8 @@ def test_the_librarys_tuned_plans_go_to_a_file_and_come_back(tmp_path):
     assert ops.library_plans_load(str(other), DEV) == 0
     other.write_text(json.dumps(dict(doc, plans=[[m3, n, k, k, k, n, 1 << 30, 12.5, 0]])))  # no such algorithm
     assert ops.library_plans_load(str(other), DEV) == 0
+    other.write_text(json.dumps(dict(doc, plans=[[-5, n, k, k, k, n, index, 12.5, 0], [m3, n, k, 1, 1, 1, index, 1.0, 0]])))
+    assert ops.library_plans_load(str(other), DEV) == 0  # sizes and strides that cannot be: skipped, no error
     other.write_text("{ not json")
     assert ops.library_plans_load(str(other), DEV) == 0
     assert ops.library_plans_load(str(tmp_path / "missing.json"), DEV) == 0
