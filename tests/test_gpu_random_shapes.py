@@ -127,3 +127,33 @@ def test_generation_with_engine_settings_drawn_at_random(tmp_path, seed):
                 assert row[token] >= row.max() - slack, f"{what}: {dtype}, request {i}, token {j} is not the arg-max"
         engine.runner.cache.check()
         del engine
+
+
+@pytest.mark.parametrize("hidden,inter,vocab", [(100, 150, 333), (36, 50, 101), (66, 130, 99), (7, 6, 11)])
+def test_widths_that_are_no_multiple_of_eight(tmp_path, hidden, inter, vocab):
+    """Widths that no 16-byte access divides (100, 36, 66, even 7 with a feed-forward of 6 and 11 tokens in the
+    vocabulary): whichever kernels take them, both dtypes, whole sequences and mixed steps."""
+    import tiny_models
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.engine.runner import ModelRunner
+    from rvllm_amd.models.registry import architecture_of
+    import rvllm_amd.models.gemma3  # noqa: F401
+    from rvllm_amd.weights.random_init import write_random_model
+
+    doc = dict(tiny_models.CONFIG_A, hidden_size=hidden, intermediate_size=inter, vocab_size=vocab)
+    config = architecture_of(doc).read_config(doc, "a narrow configuration")
+    folder = write_random_model(tmp_path / "model", config, 1, torch.bfloat16)
+    (folder / "config.json").write_text(json.dumps(doc))
+    weights, cfg = plain_gemma.load_weights(folder), plain_gemma.read_config(folder)
+    seqs = tt.make_sequences(vocab, [70, 9, 33], seed=1)
+    want = {name: plain_gemma.forward(weights, cfg, ids, torch.float64) for name, ids in seqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        for steps in (tt.trace_whole(seqs), tt.trace_mixed(seqs, seed=1)):
+            runner = ModelRunner.from_model_dir(folder, EngineConfig(
+                dtype=dtype, max_model_len=128, max_num_seqs=4, max_num_batched_tokens=128, max_prefill_chunk=128,
+                max_cache_tokens=256))
+            got = tt.collect(steps, tt.run_in_process(runner, steps), vocab)
+            assert len(got) == len(seqs)
+            for rid, logits in got.items():
+                tt.compare(logits, want[rid.split("-", 1)[1]], dtype, f"{hidden} wide, {dtype}, {rid}")
+            del runner
