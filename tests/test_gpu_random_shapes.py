@@ -157,3 +157,54 @@ def test_widths_that_are_no_multiple_of_eight(tmp_path, hidden, inter, vocab):
             for rid, logits in got.items():
                 tt.compare(logits, want[rid.split("-", 1)[1]], dtype, f"{hidden} wide, {dtype}, {rid}")
             del runner
+
+
+@pytest.mark.parametrize("nq,nkv,hd", [(1, 1, 16), (64, 1, 32), (2, 2, 512), (40, 2, 64), (3, 1, 24)])
+def test_head_counts_and_sizes_at_the_edges(tmp_path, nq, nkv, hd):
+    """One head; 64 and 20 query heads on a key/value head (more than the matrix-core kernels take); the largest
+    head size there is a kernel for; a head size that is no multiple of 16: both dtypes, whole and mixed."""
+    import tiny_models
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.engine.runner import ModelRunner
+    from rvllm_amd.models.registry import architecture_of
+    import rvllm_amd.models.gemma3  # noqa: F401
+    from rvllm_amd.weights.random_init import write_random_model
+
+    doc = dict(tiny_models.CONFIG_A, num_attention_heads=nq, num_key_value_heads=nkv, head_dim=hd,
+               query_pre_attn_scalar=hd)
+    config = architecture_of(doc).read_config(doc, "heads at the edges")
+    folder = write_random_model(tmp_path / "model", config, 1, torch.bfloat16)
+    (folder / "config.json").write_text(json.dumps(doc))
+    weights, cfg = plain_gemma.load_weights(folder), plain_gemma.read_config(folder)
+    seqs = tt.make_sequences(doc["vocab_size"], [70, 9, 33], seed=1)
+    want = {name: plain_gemma.forward(weights, cfg, ids, torch.float64) for name, ids in seqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        for steps in (tt.trace_whole(seqs), tt.trace_mixed(seqs, seed=1)):
+            runner = ModelRunner.from_model_dir(folder, EngineConfig(
+                dtype=dtype, max_model_len=128, max_num_seqs=4, max_num_batched_tokens=128, max_prefill_chunk=128,
+                max_cache_tokens=256))
+            got = tt.collect(steps, tt.run_in_process(runner, steps), doc["vocab_size"])
+            assert len(got) == len(seqs)
+            for rid, logits in got.items():
+                tt.compare(logits, want[rid.split("-", 1)[1]], dtype, f"{nq}:{nkv} heads of {hd}, {dtype}, {rid}")
+            del runner
+
+
+def test_a_head_size_beyond_the_kernels_is_refused_by_name(tmp_path):
+    import tiny_models
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.engine.runner import ModelRunner
+    from rvllm_amd.kernels import ops
+    from rvllm_amd.models.registry import architecture_of
+    import rvllm_amd.models.gemma3  # noqa: F401
+    from rvllm_amd.weights.random_init import write_random_model
+
+    doc = dict(tiny_models.CONFIG_A, num_attention_heads=2, num_key_value_heads=1, head_dim=528)
+    config = architecture_of(doc).read_config(doc, "a head too large")
+    folder = write_random_model(tmp_path / "model", config, 1, torch.bfloat16)
+    (folder / "config.json").write_text(json.dumps(doc))
+    for dtype in ("float32", "bfloat16"):
+        runner = ModelRunner.from_model_dir(folder, EngineConfig(dtype=dtype, max_model_len=64, max_num_seqs=1))
+        runner.add_request("x")
+        with pytest.raises(ops.KernelError, match="head_dim 528"):
+            runner.step([("x", [1, 2, 3], [2])])
